@@ -127,6 +127,8 @@ int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, i
                  ktx_stream_t stream);
 
 enum { KTX_GG_TILE_M = 64, KTX_GG_TILE_M_WIDE = 128 };
+/* epilogues of the grouped products: none; silu(gate) * up over a [2N][K] matrix (streaming form only); relu(y)^2 */
+enum { KTX_GG_ACT_NONE = 0, KTX_GG_ACT_GLU_SILU = 1, KTX_GG_ACT_RELU_SQ = 2 };
 
 /* Grouped GEMM  Y_g = A_g W_g^T  on the matrix cores (the product runs in W's type like ktx_dense_gemm; Y fp32 or bf16).
  * W: G matrices [N][K] back to back.
@@ -134,17 +136,20 @@ enum { KTX_GG_TILE_M = 64, KTX_GG_TILE_M_WIDE = 128 };
  *   y_goff * g .. of Y's rows (per-head products of a [T][heads][.] tensor).
  * Ragged form: sorted rows group_off[g] .. group_off[g+1] belong to group g; the A row of sorted row r is a_rows[r] (NULL: r itself), its
  *   Y row is r; tiles come from ktx_moe_plan (max_tiles bounds the launch, num_tiles[0] on the device says how many are real) and hold
- *   tile_m = 64 rows, or 128 (bf16 products only: the wide tile prompts take). */
+ *   tile_m = 64 rows, or 128 (bf16 products only: the wide tile prompts take).  The plan may hold MORE groups than G (a router whose
+ *   last outputs stand for experts without weights): their tiles are skipped and their Y rows left untouched.
+ * act: KTX_GG_ACT_NONE or KTX_GG_ACT_RELU_SQ, applied to Y. */
 int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, int64_t a_goff, const int32_t* d_a_rows,
                      const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
                      const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles, int tile_m,
-                     ktx_stream_t stream);
+                     int act, ktx_stream_t stream);
 
 /* The ragged products for a handful of rows (decode steps), streaming each row's weights once: Y[r] = W_g A[a_rows ? a_rows[r] : r]
- * with g = row_group[r].  glu != 0: W_g is [2N][K] (gate rows, then up rows) and Y[r][n] = silu(gate_n . a) * (up_n . a) — the
- * activation of a GLU expert in the same launch.  fp32 accumulation on the vector ALUs; any N, K. */
+ * with g = row_group[r]; rows whose group is >= G (no weights) are left untouched.  act = KTX_GG_ACT_GLU_SILU: W_g is [2N][K] (gate
+ * rows, then up rows) and Y[r][n] = silu(gate_n . a) * (up_n . a) — the activation of a GLU expert in the same launch;
+ * KTX_GG_ACT_RELU_SQ: Y = relu(Y)^2.  fp32 accumulation on the vector ALUs; any N, K. */
 int ktx_grouped_gemv(int R, int N, int K, const void* d_A, int a_dtype, int64_t lda, const int32_t* d_a_rows, const void* d_W, int w_dtype,
-                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int glu, ktx_stream_t stream);
+                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int act, int G, ktx_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -39,8 +39,8 @@ lib.ktx_latattn_mfma_eligible.argtypes = [C.POINTER(_LatAttnConfig)]
 lib.ktx_latattn_mfma.argtypes = [C.POINTER(_LatAttnConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_moe_route.argtypes = [_I, _I, _I, _F, _F, _P, _L, _P, _P, _P]
 lib.ktx_moe_plan.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]
-lib.ktx_grouped_gemv.argtypes = [_I, _I, _I, _P, _I, _L, _P, _P, _I, _P, _I, _L, _P, _I, _P]
-lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _I, _P]
+lib.ktx_grouped_gemv.argtypes = [_I, _I, _I, _P, _I, _L, _P, _P, _I, _P, _I, _L, _P, _I, _I, _P]
+lib.ktx_grouped_gemm.argtypes = [_I, _I, _I, _I, _P, _I, _L, _L, _P, _P, _I, _P, _I, _L, _L, _P, _P, _P, _P, _I, _I, _I, _P]
 
 TILE_M = 64
 TILE_M_WIDE, WIDE_MIN_ROWS_PER_EXPERT = 128, 96      # bf16 steps whose experts average this many rows take 128-row tiles
@@ -285,24 +285,33 @@ def head_gemm(a: torch.Tensor, a_goff: int, w: torch.Tensor, out: torch.Tensor, 
     _gg_types(a, w, out.dtype)
     M = a.shape[0]
     check(lib.ktx_grouped_gemm(G, M, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), a_goff, None, w.data_ptr(), SEQ_DTYPE[w.dtype],
-                               out.data_ptr(), SEQ_DTYPE[out.dtype], out.stride(0), y_goff, None, None, None, None, 0, TILE_M, _stream_ptr(a.device)))
+                               out.data_ptr(), SEQ_DTYPE[out.dtype], out.stride(0), y_goff, None, None, None, None, 0, TILE_M, 0, _stream_ptr(a.device)))
     return out
 
 
 GEMV_MAX_ROWS = 64      # up to this many (token, choice) pairs a step's expert products stream the weights per row instead of tiling
 
 
-def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, out_dtype=torch.float32, glu: bool = False) -> torch.Tensor:
-    """Sorted row r (expert g = the group it falls in) : out[r] = a[plan.sorted_tok[r] if gather else r] @ w[g]^T.  w [E, N, K].
-    glu (only for steps of at most GEMV_MAX_ROWS pairs): w[g] = [gate ; up] and out[r] = silu(gate a) * (up a), [pairs, N / 2]."""
+GG_ACT = {None: 0, "none": 0, "glu_silu": 1, "relu_sq": 2}
+
+
+def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, out_dtype=torch.float32, glu: bool = False,
+                act: str | None = None) -> torch.Tensor:
+    """Sorted row r (expert g = the group it falls in) : out[r] = a[plan.sorted_tok[r] if gather else r] @ w[g]^T.  w [E, N, K]; rows
+    of groups >= E (a plan over more groups than there are weights) are left as they are.
+    glu (only for steps of at most GEMV_MAX_ROWS pairs): w[g] = [gate ; up] and out[r] = silu(gate a) * (up a), [pairs, N / 2].
+    act = "relu_sq": out = relu(out)^2 in the product's epilogue."""
     G, N, K = w.shape
     _gg_types(a, w, out_dtype)
+    if glu and act:
+        raise KtxError("expert_gemm: one epilogue")
     if plan.pairs <= GEMV_MAX_ROWS:
         n_out = N // 2 if glu else N
         out = torch.empty((plan.pairs, n_out), dtype=out_dtype, device=a.device)
         check(lib.ktx_grouped_gemv(plan.pairs, n_out, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0),
                                    plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
-                                   SEQ_DTYPE[out_dtype], out.stride(0), plan.sorted_group.data_ptr(), int(glu), _stream_ptr(a.device)))
+                                   SEQ_DTYPE[out_dtype], out.stride(0), plan.sorted_group.data_ptr(), 1 if glu else GG_ACT[act], G,
+                                   _stream_ptr(a.device)))
         return out
     if glu:
         raise KtxError("expert_gemm: the fused activation is the streaming form's (at most GEMV_MAX_ROWS pairs)")
@@ -310,5 +319,5 @@ def expert_gemm(a: torch.Tensor, w: torch.Tensor, plan: MoePlan, gather: bool, o
     check(lib.ktx_grouped_gemm(G, plan.pairs, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), 0,
                                plan.sorted_tok.data_ptr() if gather else None, w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
                                SEQ_DTYPE[out_dtype], out.stride(0), 0, plan.group_off.data_ptr(), plan.tile_group.data_ptr(),
-                               plan.tile_row0.data_ptr(), plan.num_tiles.data_ptr(), plan.max_tiles, plan.tile_m, _stream_ptr(a.device)))
+                               plan.tile_row0.data_ptr(), plan.num_tiles.data_ptr(), plan.max_tiles, plan.tile_m, GG_ACT[act], _stream_ptr(a.device)))
     return out

@@ -18,10 +18,10 @@ CSRC = os.path.join(HERE, "csrc")
 LIBDIR = os.path.join(HERE, "lib")
 OBJDIR = os.path.join(LIBDIR, "obj")
 LIB = os.path.join(LIBDIR, "libktx_hip.so")
-# the sequence-mixer and hybrid-decoder kernels alone (include/ktx_seq.h, ktx_hyb.h): what the fp32-residual families need, built in
+# the sequence-mixer, hybrid-decoder and window-attention / scan kernels alone (include/ktx_seq.h, ktx_hyb.h, ktx_swa.h): what the fp32-residual families need, built in
 # well under a minute
 SEQ_LIB = os.path.join(LIBDIR, "libktx_seq.so")
-SEQ_SOURCES = ("ktx_seq.hip", "ktx_hyb.hip", "ktx_err.hip")
+SEQ_SOURCES = ("ktx_seq.hip", "ktx_hyb.hip", "ktx_swa.hip", "ktx_err.hip")
 
 # -ffp-contract=off: the parity contract needs every fp32 op rounded exactly as the reference's AVX512 code does;
 # FMAs appear only where the reference issues one (explicit fmaf()).
@@ -31,7 +31,7 @@ CFLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-f
 # per-source extra flags: the sequence-mixer kernels keep fp32 state and norms on the vector ALUs and are built without the packed
 # fp32 instructions (scalar v_fma / v_mul only)
 _NO_PACKED_FP32 = ["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
-EXTRA_CFLAGS = {"ktx_seq.hip": _NO_PACKED_FP32, "ktx_hyb.hip": _NO_PACKED_FP32}
+EXTRA_CFLAGS = {"ktx_seq.hip": _NO_PACKED_FP32, "ktx_hyb.hip": _NO_PACKED_FP32, "ktx_swa.hip": _NO_PACKED_FP32}
 
 
 def sources() -> list[str]:
@@ -82,12 +82,16 @@ def build_seq(force: bool = False, verbose: bool = False) -> str:
         return SEQ_LIB
     os.makedirs(OBJDIR, exist_ok=True)
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    for src in srcs:
-        if force or _stale(_obj(src), [src] + _deps(src)):
-            cmd = [hipcc, *CFLAGS, *EXTRA_CFLAGS.get(os.path.basename(src), []), "-c", src, "-o", _obj(src)]
-            if verbose:
-                print(" ".join(cmd), file=sys.stderr)
-            subprocess.run(cmd, check=True)
+
+    def compile_one(src: str) -> None:
+        cmd = [hipcc, *CFLAGS, *EXTRA_CFLAGS.get(os.path.basename(src), []), "-c", src, "-o", _obj(src)]
+        if verbose:
+            print(" ".join(cmd), file=sys.stderr)
+        subprocess.run(cmd, check=True)
+
+    todo = [s for s in srcs if force or _stale(_obj(s), [s] + _deps(s))]
+    with ThreadPoolExecutor(max_workers=max(1, min(len(todo), os.cpu_count() or 4))) as ex:
+        list(ex.map(compile_one, todo))
     tmp = SEQ_LIB + f".tmp{os.getpid()}"
     subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *[_obj(s) for s in srcs], "-o", tmp], check=True)
     os.replace(tmp, SEQ_LIB)

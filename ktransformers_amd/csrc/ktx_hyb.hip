@@ -844,13 +844,22 @@ __device__ __forceinline__ void gg_stage_rows(CT* dst, const AT* __restrict__ sr
   }
 }
 
+// epilogue of the grouped products: KTX_GG_ACT_RELU_SQ squares the positive part
+__device__ __forceinline__ float gg_act(float v, int act) {
+  if (act == KTX_GG_ACT_RELU_SQ) {
+    const float r = fmaxf(v, 0.f);
+    return r * r;
+  }
+  return v;
+}
+
 template <typename AT, typename CT, typename YT>
 __global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda, int64_t a_goff,
                                                            const int32_t* __restrict__ a_rows, const CT* __restrict__ W,
                                                            YT* __restrict__ Y, int64_t ldy, int64_t y_goff,
                                                            const int32_t* __restrict__ group_off, const int32_t* __restrict__ tile_group,
                                                            const int32_t* __restrict__ tile_row0, const int32_t* __restrict__ num_tiles,
-                                                           bool vec_a, bool vec_w) {
+                                                           bool vec_a, bool vec_w, int G, int act) {
   constexpr int LD = GemmTraits<CT>::LDS_LD;
   __shared__ __attribute__((aligned(16))) CT As[64 * LD];
   __shared__ __attribute__((aligned(16))) CT Ws[64 * LD];
@@ -858,6 +867,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, 
   if (group_off) {
     if ((int)blockIdx.y >= num_tiles[0]) return;
     g = tile_group[blockIdx.y];
+    if (g >= G) return;                  // a group without weights (its rows are the caller's to fill)
     m0 = tile_row0[blockIdx.y];
     m_end = group_off[g + 1];
   } else {
@@ -916,7 +926,7 @@ __global__ void __launch_bounds__(256) grouped_gemm_kernel(int M, int N, int K, 
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
-        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, acc[i][j][r]);
+        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, gg_act(acc[i][j][r], act));
       }
 }
 
@@ -927,12 +937,15 @@ __global__ void __launch_bounds__(256) grouped_gemm128_kernel(int N, int K, cons
                                                               const int32_t* __restrict__ a_rows, const bf16_t* __restrict__ W,
                                                               YT* __restrict__ Y, int64_t ldy, const int32_t* __restrict__ group_off,
                                                               const int32_t* __restrict__ tile_group, const int32_t* __restrict__ tile_row0,
-                                                              const int32_t* __restrict__ num_tiles, bool vec_a, bool vec_w) {
+                                                              const int32_t* __restrict__ num_tiles, bool vec_a, bool vec_w, int G,
+                                                              int act) {
   constexpr int LD = GemmTraits<bf16_t>::LDS_LD;
   __shared__ __attribute__((aligned(16))) bf16_t As[128 * LD];
   __shared__ __attribute__((aligned(16))) bf16_t Ws[128 * LD];
   if ((int)blockIdx.y >= num_tiles[0]) return;
-  const int g = tile_group[blockIdx.y], m0 = tile_row0[blockIdx.y], m_end = group_off[g + 1];
+  const int g = tile_group[blockIdx.y];
+  if (g >= G) return;
+  const int m0 = tile_row0[blockIdx.y], m_end = group_off[g + 1];
   const bf16_t* Wg = W + (size_t)g * N * K;
   const int n0 = blockIdx.x * 128;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -968,7 +981,7 @@ __global__ void __launch_bounds__(256) grouped_gemm128_kernel(int N, int K, cons
 #pragma unroll
       for (int r = 0; r < 4; r++) {
         const int m = m0 + wm + i * 16 + lq * 4 + r, n = n0 + wn + j * 16 + l16;
-        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, acc[i][j][r]);
+        if (m < m_end && n < N) st_elem(Y, (size_t)m * ldy + n, gg_act(acc[i][j][r], act));
       }
 }
 
@@ -979,8 +992,10 @@ template <typename AT, typename CT, typename YT>
 __global__ void __launch_bounds__(256) grouped_gemv_kernel(int N, int K, const AT* __restrict__ A, int64_t lda,
                                                            const int32_t* __restrict__ a_rows, const CT* __restrict__ W, int w_rows,
                                                            YT* __restrict__ Y, int64_t ldy, const int32_t* __restrict__ row_group,
-                                                           int glu, bool vec) {
+                                                           int act, bool vec, int G) {
   const int r = blockIdx.y, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  if (row_group[r] >= G) return;         // a group without weights
+  const bool glu = act == KTX_GG_ACT_GLU_SILU;
   const AT* a = A + (size_t)(a_rows ? a_rows[r] : r) * lda;
   const CT* Wg = W + (size_t)row_group[r] * w_rows * K;
 #pragma unroll
@@ -1034,7 +1049,7 @@ __global__ void __launch_bounds__(256) grouped_gemv_kernel(int N, int K, const A
     }
     s0 = wave_sum(s0);
     if (glu) s1 = wave_sum(s1);
-    if (lane == 0) st_elem(Y, (size_t)r * ldy + n, glu ? silu_f32(s0) * s1 : s0);
+    if (lane == 0) st_elem(Y, (size_t)r * ldy + n, glu ? silu_f32(s0) * s1 : gg_act(s0, act));
   }
 }
 
@@ -1317,8 +1332,9 @@ int ktx_moe_plan(int T, int E, int top, int tile_m, const int32_t* d_topk_idx, i
 int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, int64_t a_goff, const int32_t* d_a_rows,
                      const void* d_W, int w_dtype, void* d_Y, int y_dtype, int64_t ldy, int64_t y_goff, const int32_t* d_group_off,
                      const int32_t* d_tile_group, const int32_t* d_tile_row0, const int32_t* d_num_tiles, int max_tiles, int tile_m,
-                     ktx_stream_t stream) {
+                     int act, ktx_stream_t stream) {
   KTX_REQUIRE(G > 0 && M >= 0 && N > 0 && K > 0 && d_A && d_W && d_Y, "ktx_grouped_gemm: G, N, K > 0, pointers");
+  KTX_REQUIRE(act == KTX_GG_ACT_NONE || act == KTX_GG_ACT_RELU_SQ, "ktx_grouped_gemm: epilogue none or relu^2");
   KTX_REQUIRE(dtype_ok(a_dtype) && dtype_ok(w_dtype) && dtype_ok(y_dtype), "ktx_grouped_gemm: unknown element type");
   KTX_REQUIRE(!(w_dtype == KTX_SEQ_F32 && (a_dtype != KTX_SEQ_F32 || y_dtype != KTX_SEQ_F32)),
               "ktx_grouped_gemm: an fp32 product takes and writes fp32");
@@ -1337,7 +1353,7 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
     hipStream_t st1 = (hipStream_t)stream;
 #define KTX_GG128_GO(AT, YT)                                                                                                       \
   grouped_gemm128_kernel<AT, YT><<<grid128, 256, 0, st1>>>(N, K, (const AT*)d_A, lda, d_a_rows, (const bf16_t*)d_W, (YT*)d_Y, ldy, \
-                                                           d_group_off, d_tile_group, d_tile_row0, d_num_tiles, va, vw)
+                                                           d_group_off, d_tile_group, d_tile_row0, d_num_tiles, va, vw, G, act)
     if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GG128_GO(float, float);
     else if (a_dtype == KTX_SEQ_F32) KTX_GG128_GO(float, bf16_t);
     else if (y_dtype == KTX_SEQ_F32) KTX_GG128_GO(bf16_t, float);
@@ -1355,7 +1371,7 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
   hipStream_t st = (hipStream_t)stream;
 #define KTX_GG_GO(AT, CT, YT)                                                                                                  \
   grouped_gemm_kernel<AT, CT, YT><<<grid, 256, 0, st>>>(M, N, K, (const AT*)d_A, lda, a_goff, d_a_rows, (const CT*)d_W, (YT*)d_Y, ldy, \
-                                                        y_goff, d_group_off, d_tile_group, d_tile_row0, d_num_tiles, vec_a, vec_w)
+                                                        y_goff, d_group_off, d_tile_group, d_tile_row0, d_num_tiles, vec_a, vec_w, G, act)
   if (w_dtype == KTX_SEQ_BF16) {
     if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GG_GO(float, bf16_t, float);
     else if (a_dtype == KTX_SEQ_F32) KTX_GG_GO(float, bf16_t, bf16_t);
@@ -1370,8 +1386,10 @@ int ktx_grouped_gemm(int G, int M, int N, int K, const void* d_A, int a_dtype, i
 }
 
 int ktx_grouped_gemv(int R, int N, int K, const void* d_A, int a_dtype, int64_t lda, const int32_t* d_a_rows, const void* d_W, int w_dtype,
-                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int glu, ktx_stream_t stream) {
-  KTX_REQUIRE(R >= 0 && N > 0 && K > 0 && d_A && d_W && d_Y && d_row_group, "ktx_grouped_gemv: N, K > 0, pointers");
+                     void* d_Y, int y_dtype, int64_t ldy, const int32_t* d_row_group, int act, int G, ktx_stream_t stream) {
+  KTX_REQUIRE(R >= 0 && N > 0 && K > 0 && G > 0 && d_A && d_W && d_Y && d_row_group, "ktx_grouped_gemv: N, K, G > 0, pointers");
+  KTX_REQUIRE(act == KTX_GG_ACT_NONE || act == KTX_GG_ACT_GLU_SILU || act == KTX_GG_ACT_RELU_SQ, "ktx_grouped_gemv: unknown epilogue");
+  const int glu = act == KTX_GG_ACT_GLU_SILU;
   KTX_REQUIRE(dtype_ok(a_dtype) && dtype_ok(w_dtype) && dtype_ok(y_dtype), "ktx_grouped_gemv: unknown element type");
   KTX_REQUIRE(R <= 65535, "ktx_grouped_gemv: up to 65535 rows");
   if (R == 0) return 0;
@@ -1382,7 +1400,7 @@ int ktx_grouped_gemv(int R, int N, int K, const void* d_A, int a_dtype, int64_t 
   hipStream_t st = (hipStream_t)stream;
 #define KTX_GV_GO(AT, CT, YT)                                                                                                          \
   grouped_gemv_kernel<AT, CT, YT><<<grid, 256, 0, st>>>(N, K, (const AT*)d_A, lda, d_a_rows, (const CT*)d_W, w_rows, (YT*)d_Y, ldy, \
-                                                        d_row_group, glu, vec)
+                                                        d_row_group, act, vec, G)
   if (w_dtype == KTX_SEQ_BF16) {
     if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GV_GO(float, bf16_t, float);
     else if (a_dtype == KTX_SEQ_F32) KTX_GV_GO(float, bf16_t, bf16_t);

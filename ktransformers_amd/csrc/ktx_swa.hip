@@ -1,0 +1,999 @@
+// ktx_swa.hip — kernels behind include/ktx_swa.h: the residual update with a scalar-weight RMS norm and the rows an input convolution
+// reads, the input convolution over time, grouped-query sliding-window attention over paged key and value caches with rotated values
+// and a sink (prep, a vector-ALU form for any sizes, a matrix-core form for bf16 caches, the key-range merge), the selective scan with
+// its short convolution, and the softmax router with a choice correction.
+//
+// Everything a norm, an angle, a score, a router or a recurrence touches is fp32; element types only select how weights, activations
+// and the caches are stored and which MFMA multiplies them.
+#include "ktx_common.h"
+#include "../../include/ktx_swa.h"
+
+#include <math.h>
+
+#include <algorithm>
+
+namespace {
+
+#include "ktx_seq_dev.inc"
+
+__device__ __forceinline__ float silu_f32(float z) { return z / (1.0f + expf(-z)); }
+__device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+bool aligned16(const void* p) { return ((uintptr_t)p & 15u) == 0; }
+int dtype_ok(int d) { return d == KTX_SEQ_F32 || d == KTX_SEQ_BF16; }
+
+// ---------------------------------------------------------------------------------------------------------------------
+// one row per workgroup; the row lives in LDS between the passes
+template <typename OT, typename HT>
+__global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restrict__ x, ktx_resid_args a) {
+  extern __shared__ float row[];
+  __shared__ float red[4];
+  const int i = blockIdx.x, tid = threadIdx.x;
+  const int t = a.rows ? a.rows[i] : i;
+  float* xr = x + (size_t)t * W;
+  const bool adds = a.y || a.ey;
+  if (adds) {
+    for (int e = tid; e < W; e += 256) row[e] = 0.f;
+    if (a.y) {
+      const float* y = a.y + (size_t)t * a.ldy;
+      float r = 1.0f;
+      if (a.y_norm_w) {
+        float s = 0.f;
+        for (int e = tid; e < W; e += 256) s += y[e] * y[e];
+        r = 1.0f / sqrtf(block_sum256(s, red) / (float)W + a.y_norm_eps);
+      }
+      for (int e = tid; e < W; e += 256) row[e] = a.y_norm_w ? y[e] * r * a.y_norm_w[e] : y[e];
+    }
+    if (a.ey) {
+      const HT* h = reinterpret_cast<const HT*>(a.h_in) + (size_t)t * W;
+      for (int k = 0; k < a.top; k++) {
+        const int g = a.topk_idx[(size_t)t * a.top + k];
+        const float w = a.topk_w[(size_t)t * a.top + k];
+        if (g < a.n_real) {
+          const float* src = a.ey + (size_t)a.pair_pos[(size_t)t * a.top + k] * W;
+          for (int e = tid; e < W; e += 256) row[e] += w * src[e];
+        } else {
+          for (int e = tid; e < W; e += 256) row[e] += w * ld_elem(h, e);
+        }
+      }
+    }
+    for (int e = tid; e < W; e += 256) {
+      const float v = xr[e] + row[e];
+      row[e] = v;
+      xr[e] = v;
+    }
+  } else {
+    for (int e = tid; e < W; e += 256) row[e] = xr[e];
+  }
+  if (!a.norm_g) return;
+  float s = 0.f;
+  for (int e = tid; e < W; e += 256) s += row[e] * row[e];
+  const float r = a.norm_g[0] / sqrtf(block_sum256(s, red) / (float)W + a.eps);
+  OT* out = reinterpret_cast<OT*>(a.out);
+  if (a.halo <= 0) {
+    for (int e = tid; e < W; e += 256) st_elem(out, (size_t)i * W + e, row[e] * r);
+    return;
+  }
+  const int b = a.tok_req[t];
+  for (int e = tid; e < W; e += 256) st_elem(out, ((size_t)t + (size_t)(b + 1) * a.halo) * W + e, row[e] * r);
+  if (t == a.q_indptr[b]) {      // the request's first new token also lays the rows in front of it
+    const bool cont = a.pos0[b] > 0;
+    const float* st = a.conv_state + (size_t)a.slot[b] * a.halo * W;
+    for (int e = tid; e < a.halo * W; e += 256) st_elem(out, ((size_t)t + (size_t)b * a.halo) * W + e, cont ? st[e] : 0.f);
+  }
+}
+
+// thread = (token, channel)
+template <typename OT>
+__global__ void __launch_bounds__(256) input_conv_kernel(int W, int taps, const float* __restrict__ hx, const float* __restrict__ w,
+                                                         const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ slot,
+                                                         const int32_t* __restrict__ tok_req, float* __restrict__ conv_state,
+                                                         OT* __restrict__ out) {
+  const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= W) return;
+  const int halo = taps - 1, b = tok_req[t];
+  const size_t r = (size_t)t + (size_t)(b + 1) * halo;
+  float acc = 0.f;
+  for (int j = 0; j < taps; j++) acc += w[(size_t)c * taps + j] * hx[(r - halo + j) * W + c];
+  st_elem(out, (size_t)t * W + c, hx[r * W + c] + acc);
+  if (t == q_indptr[b + 1] - 1) {
+    float* st = conv_state + (size_t)slot[b] * halo * W;
+    for (int i = 0; i < halo; i++) st[(size_t)i * W + c] = hx[(r - halo + 1 + i) * W + c];
+  }
+}
+
+template <typename TT, typename OT>
+__global__ void __launch_bounds__(256) rows_mul_lookup_kernel(size_t total, int n, const float* __restrict__ a, int64_t lda,
+                                                              const TT* __restrict__ table, int64_t ldt, int col0,
+                                                              const int32_t* __restrict__ tokens, OT* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= total) return;
+  const size_t t = i / n;
+  const int c = (int)(i % n);
+  st_elem(out, i, a[t * lda + c] * ld_elem(table, (size_t)tokens[t] * ldt + col0 + c));
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// attention prep: one token per workgroup, a wavefront per head
+template <typename KT>
+__global__ void __launch_bounds__(256) swa_prep_kernel(ktx_swa_config c, const float* __restrict__ proj, int64_t ldp, int q_off, int k_off,
+                                                       int v_off, const double* __restrict__ inv_freq, const double* __restrict__ v_inv_freq,
+                                                       const int32_t* __restrict__ pos, const int32_t* __restrict__ cache_loc,
+                                                       KT* __restrict__ kcache, KT* __restrict__ vcache, float* __restrict__ q_out,
+                                                       float* __restrict__ vcs) {
+  extern __shared__ float cs[];            // cos | sin of the rot_dims / 2 key angles, then cos | sin of the vdim / 2 value angles
+  const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int NP = c.rot_dims / 2, NV = c.rot_values ? c.vdim / 2 : 0;
+  float* vc = cs + 2 * NP;
+  const double p = (double)pos[t];
+  for (int i = tid; i < NP; i += 256) {
+    const double a = p * inv_freq[i];
+    cs[i] = (float)cos(a);
+    cs[NP + i] = (float)sin(a);
+  }
+  for (int i = tid; i < NV; i += 256) {
+    const double a = p * v_inv_freq[i];
+    const float co = (float)cos(a), si = (float)sin(a);
+    vc[i] = co;
+    vc[NV + i] = si;
+    vcs[(size_t)t * c.vdim + i] = co;
+    vcs[(size_t)t * c.vdim + NV + i] = si;
+  }
+  __syncthreads();
+  // entry j of a vector whose first 2 * np entries turn in pairs (2i, 2i + 1)
+  auto turned = [](const float* v, int j, int np, const float* tab) -> float {
+    if (j >= 2 * np) return v[j];
+    const int i = j >> 1;
+    const float a = v[2 * i], bb = v[2 * i + 1];
+    return (j & 1) ? bb * tab[i] + a * tab[np + i] : a * tab[i] - bb * tab[np + i];
+  };
+  const float* base = proj + (size_t)t * ldp;
+  const int D = c.dim, V = c.vdim, H = c.heads, G = c.kv_heads;
+  const size_t loc = (size_t)cache_loc[t];
+  for (int u = wave; u < H + 2 * G; u += 4) {
+    if (u < H + G) {        // a query or key head: rotate, then norm
+      const bool isq = u < H;
+      const float* v = base + (isq ? q_off + (size_t)u * D : k_off + (size_t)(u - H) * D);
+      float r = 1.0f;
+      if (c.qk_norm) {
+        float s = 0.f;
+        for (int j = lane; j < D; j += 64) {
+          const float x = turned(v, j, NP, cs);
+          s += x * x;
+        }
+        r = 1.0f / sqrtf(wave_sum(s) / (float)D + c.eps);
+      }
+      if (isq) {
+        r *= c.scale;
+        float* o = q_out + ((size_t)t * H + u) * D;
+        for (int j = lane; j < D; j += 64) o[j] = turned(v, j, NP, cs) * r;
+      } else {
+        KT* o = kcache + (loc * G + (u - H)) * D;
+        for (int j = lane; j < D; j += 64) st_elem(o, j, turned(v, j, NP, cs) * r);
+      }
+    } else {
+      const int g = u - H - G;
+      const float* v = base + v_off + (size_t)g * V;
+      KT* o = vcache + (loc * G + g) * V;
+      for (int j = lane; j < V; j += 64) st_elem(o, j, turned(v, j, NV, vc));
+    }
+  }
+}
+
+// attention of ONE token (blockIdx.x) x HG query heads of one key head (blockIdx.y) x one key range (blockIdx.z) on the vector ALUs:
+// tiles of KTN <= 64 keys and values staged in LDS as fp32; scores thread = (head, key); running maximum / sum per head by wavefronts;
+// outputs thread = (head, value entry) in registers.
+constexpr int SW_NACC = 32;
+template <typename KT, typename OT>
+__global__ void __launch_bounds__(256) swa_fwd_kernel(ktx_swa_config c, int T, int HG, int parts, int KTN, const float* __restrict__ q,
+                                                      const KT* __restrict__ kcache, const KT* __restrict__ vcache,
+                                                      const int32_t* __restrict__ tok_req, const int32_t* __restrict__ pos,
+                                                      const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_indices,
+                                                      const float* __restrict__ sink, const float* __restrict__ vcs, int nsplit,
+                                                      float* __restrict__ scratch, OT* __restrict__ out) {
+  extern __shared__ float lds[];
+  const int D = c.dim, V = c.vdim, DP = D + 1, VP = V + 1, G = c.kv_heads, HPG = c.heads / G;
+  float* qs = lds;                         // [HG][D]
+  float* kt = qs + (size_t)HG * D;         // [KTN][DP]
+  float* vt = kt + (size_t)KTN * DP;       // [KTN][VP]
+  float* sc = vt + (size_t)KTN * VP;       // [HG][KTN]
+  float* mrow = sc + (size_t)HG * KTN;     // [HG] running maximum
+  float* lrow = mrow + HG;                 // [HG] running sum
+  float* crow = lrow + HG;                 // [HG] correction of this tile
+  int* rowidx = reinterpret_cast<int*>(crow + HG);   // [KTN]
+  const int t = blockIdx.x, g = blockIdx.y / parts, part = blockIdx.y % parts, z = blockIdx.z;
+  const int h0 = g * HPG + part * HG;
+  const int nh = min(HG, HPG - part * HG);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int p = pos[t], b = tok_req[t];
+  const int jlo = c.window > 0 ? max(0, p - c.window + 1) : 0, jhi = p + 1;
+  const int per = (jhi - jlo + nsplit - 1) / nsplit;
+  const int j0 = jlo + z * per, j1 = min(jhi, j0 + per);
+  for (int e = tid; e < nh * D; e += 256) qs[e] = q[((size_t)t * c.heads + h0) * D + e];
+  for (int h = tid; h < HG; h += 256) {
+    mrow[h] = -INFINITY;
+    lrow[h] = 0.f;
+  }
+  float acc[SW_NACC];
+#pragma unroll
+  for (int i = 0; i < SW_NACC; i++) acc[i] = 0.f;
+  const int nout = nh * V;
+  const int32_t* pages = page_indices + page_indptr[b];
+  for (int jt = j0; jt < j1; jt += KTN) {
+    const int nk = min(KTN, j1 - jt);
+    __syncthreads();
+    if (tid < nk) {
+      const int j = jt + tid;
+      rowidx[tid] = pages[j / c.page_size] * c.page_size + j % c.page_size;
+    }
+    __syncthreads();
+    for (int e = tid; e < nk * D; e += 256) {
+      const int j = e / D, d = e % D;
+      kt[(size_t)j * DP + d] = ld_elem(kcache, ((size_t)rowidx[j] * G + g) * D + d);
+    }
+    for (int e = tid; e < nk * V; e += 256) {
+      const int j = e / V, d = e % V;
+      vt[(size_t)j * VP + d] = ld_elem(vcache, ((size_t)rowidx[j] * G + g) * V + d);
+    }
+    __syncthreads();
+    for (int e = tid; e < nh * KTN; e += 256) {
+      const int h = e / KTN, j = e % KTN;
+      if (j < nk) {
+        const float* qh = qs + (size_t)h * D;
+        const float* kj = kt + (size_t)j * DP;
+        float s = 0.f;
+        for (int d = 0; d < D; d++) s += qh[d] * kj[d];
+        sc[(size_t)h * KTN + j] = s;      // (scale is folded into q)
+      }
+    }
+    __syncthreads();
+    for (int h = wave; h < nh; h += 4) {
+      const float s = lane < nk ? sc[(size_t)h * KTN + lane] : -INFINITY;
+      const float mo = mrow[h];
+      const float mn = fmaxf(mo, wave_max(s));
+      const float w = lane < nk ? expf(s - mn) : 0.f;
+      const float sum = wave_sum(w);
+      if (lane < nk) sc[(size_t)h * KTN + lane] = w;
+      if (lane == 0) {
+        const float cr = mo == -INFINITY ? 0.f : expf(mo - mn);
+        crow[h] = cr;
+        mrow[h] = mn;
+        lrow[h] = lrow[h] * cr + sum;
+      }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < SW_NACC; i++) {
+      const int e = tid + i * 256;
+      if (e < nout) {
+        const int h = e / V, l = e % V;
+        float a = acc[i] * crow[h];
+        const float* w = sc + (size_t)h * KTN;
+        for (int j = 0; j < nk; j++) a += w[j] * vt[(size_t)j * VP + l];
+        acc[i] = a;
+      }
+    }
+  }
+  __syncthreads();
+  if (nsplit == 1) {
+    const int NV = V / 2;
+#pragma unroll
+    for (int i = 0; i < SW_NACC; i++) {
+      const int e = tid + i * 256;
+      const bool live = e < nout;
+      const int h = live ? e / V : 0, l = live ? e % V : 0;
+      float o = 0.f;
+      if (live) {
+        const float m = mrow[h];
+        if (sink) {
+          const float sk = sink[h0 + h], M = fmaxf(m, sk);
+          const float f = m == -INFINITY ? 0.f : expf(m - M);
+          o = acc[i] * f / (lrow[h] * f + expf(sk - M));
+        } else {
+          o = lrow[h] > 0.f ? acc[i] / lrow[h] : 0.f;
+        }
+      }
+      if (c.rot_values) {      // turn the pair (2m, 2m + 1) back by the token's own angle; the partner sits in the neighbouring thread
+        const float other = __shfl_xor(o, 1);
+        if (live) {
+          const float co = vcs[(size_t)t * V + (l >> 1)], si = vcs[(size_t)t * V + NV + (l >> 1)];
+          o = (l & 1) ? o * co - other * si : o * co + other * si;
+        }
+      }
+      if (live) st_elem(out, ((size_t)t * c.heads + h0 + h) * V + l, o);
+    }
+    return;
+  }
+  float* partial = scratch + (((size_t)z * T + t) * c.heads + h0) * (V + 2);
+#pragma unroll
+  for (int i = 0; i < SW_NACC; i++) {
+    const int e = tid + i * 256;
+    if (e < nout) partial[(size_t)(e / V) * (V + 2) + e % V] = acc[i];
+  }
+  for (int h = tid; h < nh; h += 256) {
+    partial[(size_t)h * (V + 2) + V] = mrow[h];
+    partial[(size_t)h * (V + 2) + V + 1] = lrow[h];
+  }
+}
+
+// merge the key ranges of one (token, head): thread = value entry; normalise with the sink, then turn the result back
+template <typename OT>
+__global__ void __launch_bounds__(256) swa_merge_kernel(int T, int H, int V, int nsplit, int rot_values, const float* __restrict__ scratch,
+                                                        const float* __restrict__ sink, const float* __restrict__ vcs,
+                                                        OT* __restrict__ out) {
+  extern __shared__ float mw[];            // [nsplit] maxima, then [nsplit] weights exp(m_z - M) (0 for an empty range)
+  float* ws = mw + nsplit;
+  const int t = blockIdx.x, h = blockIdx.y;
+  const size_t stride = (size_t)T * H * (V + 2);
+  const float* base = scratch + ((size_t)t * H + h) * (V + 2);
+  for (int z = threadIdx.x; z < nsplit; z += 256) {
+    mw[z] = base[z * stride + V];
+    ws[z] = base[z * stride + V + 1];
+  }
+  __syncthreads();
+  float M = sink ? sink[h] : -INFINITY;
+  for (int z = 0; z < nsplit; z++) M = fmaxf(M, mw[z]);
+  float den = sink ? expf(sink[h] - M) : 0.f;
+  for (int z = 0; z < nsplit; z++) den += mw[z] == -INFINITY ? 0.f : ws[z] * expf(mw[z] - M);
+  __syncthreads();
+  for (int z = threadIdx.x; z < nsplit; z += 256) ws[z] = mw[z] == -INFINITY ? 0.f : expf(mw[z] - M);
+  __syncthreads();
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
+  const int NV = V / 2;
+  for (int l0 = 0; l0 < V; l0 += 256) {
+    const int l = l0 + threadIdx.x;
+    const bool live = l < V;
+    float a = 0.f;
+    if (live) {
+#pragma unroll 4
+      for (int z = 0; z < nsplit; z++) a = fmaf(base[z * stride + l], ws[z], a);
+      a *= inv;
+    }
+    if (rot_values) {
+      const float other = __shfl_xor(a, 1);
+      if (live) {
+        const float co = vcs[(size_t)t * V + (l >> 1)], si = vcs[(size_t)t * V + NV + (l >> 1)];
+        a = (l & 1) ? a * co - other * si : a * co + other * si;
+      }
+    }
+    if (live) st_elem(out, ((size_t)t * H + h) * V + l, a);
+  }
+}
+
+// The same attention on the matrix cores (bf16 caches).  The (token, head) pairs of a request that share key head g (blockIdx.y) are the
+// rows of one query matrix: a workgroup takes 64 consecutive rows (its four wavefronts one 16-row MFMA tile each, query fragments
+// resident in registers) and walks 32-key tiles of the union of its rows' windows: keys staged row-major, values transposed; scores,
+// mask, running maximum and sum in fp32 (DPP reductions inside the 16-lane column groups), weights through a per-wavefront LDS tile
+// into the second product.  Key ranges (blockIdx.z) leave unnormalised partial sums that swa_merge_kernel joins.
+constexpr int SM_KT = 32, SM_PST = SM_KT + 8, SM_KSMAX = 8;
+template <int NT, typename OT>
+__global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, int row_tiles, const float* __restrict__ q,
+                                                       const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
+                                                       const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                       const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_indices,
+                                                       const float* __restrict__ sink, const float* __restrict__ vcs, int nsplit,
+                                                       float* __restrict__ scratch, OT* __restrict__ out) {
+  constexpr int V = NT * 16;
+  extern __shared__ __attribute__((aligned(16))) unsigned char sm_raw[];
+  const int H = c.heads, G = c.kv_heads, HPG = H / G, D = c.dim, DPP = D + 8, KS = D / 32;
+  bf16_t* Ks = reinterpret_cast<bf16_t*>(sm_raw);            // [SM_KT][DPP]
+  bf16_t* Vt = Ks + (size_t)SM_KT * DPP;                      // [V][SM_PST]
+  bf16_t* Ps = Vt + (size_t)V * SM_PST;                       // [4][16][SM_PST]
+  int* rowidx = reinterpret_cast<int*>(Ps + 4 * 16 * SM_PST); // [SM_KT]
+  const int b = blockIdx.x / row_tiles, rt = blockIdx.x % row_tiles, g = blockIdx.y, z = blockIdx.z;
+  const int t0 = q_indptr[b], rows_total = (q_indptr[b + 1] - t0) * HPG, r0 = rt * 64;
+  if (r0 >= rows_total) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
+  const int p0 = pos0[b];
+  const int tok_lo = r0 / HPG, tok_hi = (min(rows_total, r0 + 64) - 1) / HPG;
+  const int klo = c.window > 0 ? max(0, p0 + tok_lo - c.window + 1) : 0, khi = p0 + tok_hi + 1;
+  const int per = (((khi - klo + nsplit - 1) / nsplit) + SM_KT - 1) / SM_KT * SM_KT;
+  const int j0 = klo + z * per, j1 = min(khi, j0 + per);
+  const int rw0 = r0 + wave * 16;
+  const bool active = rw0 < rows_total;
+  // query fragments: lane = (row l16, 8 consecutive entries lq * 8 ..) of every 32-entry step
+  sq_v8bf qf[SM_KSMAX];
+  {
+    const int ar = min(rw0 + l16, rows_total - 1);
+    const bool live = rw0 + l16 < rows_total;
+    const float* qrow = q + ((size_t)(t0 + ar / HPG) * H + g * HPG + ar % HPG) * D;
+#pragma unroll
+    for (int kk = 0; kk < SM_KSMAX; kk++) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; i++) v[i] = 0.f;
+      if (kk < KS && live) {
+        const int e0 = kk * 32 + lq * 8;
+        const float4 x = *reinterpret_cast<const float4*>(qrow + e0), y = *reinterpret_cast<const float4*>(qrow + e0 + 4);
+        v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w; v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+      }
+      union { uint4 u; sq_v8bf f; } cv;
+      cv.u.x = ktx_pk_bf16(v[0], v[1]); cv.u.y = ktx_pk_bf16(v[2], v[3]); cv.u.z = ktx_pk_bf16(v[4], v[5]); cv.u.w = ktx_pk_bf16(v[6], v[7]);
+      qf[kk] = cv.f;
+    }
+  }
+  // the four rows this lane holds of the score / output tiles (C layout: row lq * 4 + r, column l16)
+  int prow[4], lorow[4];
+  bool vrow[4];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int cr = rw0 + lq * 4 + r;
+    vrow[r] = cr < rows_total;
+    prow[r] = p0 + cr / HPG;
+    lorow[r] = c.window > 0 ? max(0, prow[r] - c.window + 1) : 0;
+  }
+  float mrun[4], lrun[4];
+  v4f acc[NT];
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    mrun[r] = -INFINITY;
+    lrun[r] = 0.f;
+  }
+#pragma unroll
+  for (int n = 0; n < NT; n++) acc[n] = (v4f){0.f, 0.f, 0.f, 0.f};
+  const int32_t* pages = page_indices + page_indptr[b];
+  const int ksegs = D / 8, vsegs = V / 8;
+  bf16_t* Pw = Ps + (size_t)wave * 16 * SM_PST;
+  for (int jt = j0; jt < j1; jt += SM_KT) {
+    const int nk = min(SM_KT, j1 - jt);
+    __syncthreads();
+    if (tid < SM_KT) {
+      const int j = jt + tid;
+      rowidx[tid] = tid < nk ? pages[j / c.page_size] * c.page_size + j % c.page_size : -1;
+    }
+    __syncthreads();
+    for (int idx = tid; idx < SM_KT * ksegs; idx += 256) {
+      const int key = idx / ksegs, e0 = (idx % ksegs) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      const int row = rowidx[key];
+      if (row >= 0) v = *reinterpret_cast<const uint4*>(kcache + ((size_t)row * G + g) * D + e0);
+      *reinterpret_cast<uint4*>(Ks + (size_t)key * DPP + e0) = v;
+    }
+    for (int idx = tid; idx < SM_KT * vsegs; idx += 256) {
+      const int key = idx % SM_KT, e0 = (idx / SM_KT) * 8;
+      uint4 v = make_uint4(0u, 0u, 0u, 0u);
+      const int row = rowidx[key];
+      if (row >= 0) v = *reinterpret_cast<const uint4*>(vcache + ((size_t)row * G + g) * V + e0);
+      const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int i = 0; i < 8; i++) Vt[(size_t)(e0 + i) * SM_PST + key] = (bf16_t)((w[i >> 1] >> ((i & 1) * 16)) & 0xffffu);
+    }
+    __syncthreads();
+    if (active) {
+      v4f s0 = (v4f){0.f, 0.f, 0.f, 0.f}, s1 = s0;
+#pragma unroll
+      for (int kk = 0; kk < SM_KSMAX; kk++) {
+        if (kk < KS) {
+          const sq_v8bf b0 = *reinterpret_cast<const sq_v8bf*>(Ks + (size_t)l16 * DPP + kk * 32 + lq * 8);
+          const sq_v8bf b1 = *reinterpret_cast<const sq_v8bf*>(Ks + (size_t)(16 + l16) * DPP + kk * 32 + lq * 8);
+          s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], b0, s0, 0, 0, 0);
+          s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], b1, s1, 0, 0, 0);
+        }
+      }
+      const int ja = jt + l16, jb = ja + 16;
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const bool oka = vrow[r] && ja < j1 && ja >= lorow[r] && ja <= prow[r];
+        const bool okb = vrow[r] && jb < j1 && jb >= lorow[r] && jb <= prow[r];
+        const float sa = oka ? s0[r] : -INFINITY, sb = okb ? s1[r] : -INFINITY;      // (scale is folded into q)
+        const float mt = row16_max(fmaxf(sa, sb));
+        const float mn = fmaxf(mrun[r], mt);
+        const float mb = mn == -INFINITY ? 0.f : mn;
+        const float wa = oka ? __expf(sa - mb) : 0.f, wb = okb ? __expf(sb - mb) : 0.f;
+        const float cr = mrun[r] == -INFINITY ? 0.f : __expf(mrun[r] - mb);
+        lrun[r] = lrun[r] * cr + row16_sum(wa + wb);
+        mrun[r] = mn;
+#pragma unroll
+        for (int n = 0; n < NT; n++) acc[n][r] *= cr;
+        Pw[(lq * 4 + r) * SM_PST + l16] = to_bf16_rne(wa);
+        Pw[(lq * 4 + r) * SM_PST + 16 + l16] = to_bf16_rne(wb);
+      }
+    }
+    __syncthreads();
+    if (active) {
+      const sq_v8bf pf = *reinterpret_cast<const sq_v8bf*>(Pw + (size_t)l16 * SM_PST + lq * 8);
+#pragma unroll
+      for (int n = 0; n < NT; n++) {
+        const sq_v8bf vb = *reinterpret_cast<const sq_v8bf*>(Vt + (size_t)(n * 16 + l16) * SM_PST + lq * 8);
+        acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(pf, vb, acc[n], 0, 0, 0);
+      }
+    }
+  }
+  if (!active) return;
+  constexpr int NV = V / 2;
+#pragma unroll
+  for (int r = 0; r < 4; r++) {
+    const int cr = min(rw0 + lq * 4 + r, rows_total - 1);
+    const int tok = t0 + cr / HPG, head = g * HPG + cr % HPG;
+    const size_t grow = (size_t)tok * H + head;             // (token, head) row of out
+    if (nsplit == 1) {
+      float inv;
+      if (sink) {
+        const float sk = sink[head], M = fmaxf(mrun[r], sk);
+        const float f = mrun[r] == -INFINITY ? 0.f : expf(mrun[r] - M);
+        inv = f / (lrun[r] * f + expf(sk - M));
+      } else {
+        inv = lrun[r] > 0.f ? 1.0f / lrun[r] : 0.f;
+      }
+#pragma unroll
+      for (int n = 0; n < NT; n++) {
+        float o = acc[n][r] * inv;
+        if (c.rot_values) {      // column n * 16 + l16 pairs with its neighbour column: the neighbouring lane of the quad
+          const float other = ktx_dpp_f<KTX_DPP_QUAD_1032>(o);
+          const int m = (n * 16 + l16) >> 1;
+          const float co = vcs[(size_t)tok * V + m], si = vcs[(size_t)tok * V + NV + m];
+          o = (l16 & 1) ? o * co - other * si : o * co + other * si;
+        }
+        if (vrow[r]) st_elem(out, grow * V + n * 16 + l16, o);
+      }
+    } else if (vrow[r]) {
+      float* part = scratch + ((size_t)z * T * H + grow) * (V + 2);
+#pragma unroll
+      for (int n = 0; n < NT; n++) part[n * 16 + l16] = acc[n][r];
+      if (l16 == 0) {
+        part[V] = mrun[r];
+        part[V + 1] = lrun[r];
+      }
+    }
+  }
+}
+
+size_t swa_mfma_lds(const ktx_swa_config& c) {
+  return ((size_t)SM_KT * (c.dim + 8) + (size_t)c.vdim * SM_PST + 4 * 16 * SM_PST) * 2 + SM_KT * 4;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// selective scan.  thread = (token, channel) for the convolution
+constexpr int SSM_MAX_TAPS = 8;
+__global__ void __launch_bounds__(256) ssm_conv_kernel(ktx_ssm_config c, const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                       const int32_t* __restrict__ slot, const int32_t* __restrict__ tok_req,
+                                                       const float* __restrict__ proj, int64_t ldp, int x_off, const float* __restrict__ w,
+                                                       const float* __restrict__ bias, const float* __restrict__ conv_state,
+                                                       float* __restrict__ xc) {
+  const int t = blockIdx.x, ch = blockIdx.y * 256 + threadIdx.x;
+  if (ch >= c.inner) return;
+  const int b = tok_req[t], q0 = q_indptr[b], i = t - q0, K = c.taps;
+  const bool cont = pos0[b] > 0;
+  float acc = bias ? bias[ch] : 0.f;
+  for (int j = 0; j < K; j++) {
+    const int s = i - K + 1 + j;
+    float v = 0.f;
+    if (s >= 0) v = proj[(size_t)(q0 + s) * ldp + x_off + ch];
+    else if (cont) v = conv_state[((size_t)slot[b] * (K - 1) + (K - 1 + s)) * c.inner + ch];
+    acc += w[(size_t)ch * K + j] * v;
+  }
+  xc[(size_t)t * c.inner + ch] = silu_f32(acc);
+}
+
+// The recurrence: a workgroup owns 256 / LPC channels of one request; a channel's state entries are split over LPC neighbouring lanes
+// (16 each, in registers).  Tokens are taken SS_TC at a time: the step's B and C rows of the chunk are staged in LDS once for all
+// channels, the per-channel inputs (step, x, gate) requested for the whole chunk before the sequential part starts.
+constexpr int SS_NS = 16, SS_TC = 8;
+template <int LPC, typename OT>
+__global__ void __launch_bounds__(256) ssm_scan_kernel(ktx_ssm_config c, const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                       const int32_t* __restrict__ slot, const float* __restrict__ xc,
+                                                       const float* __restrict__ Bm, const float* __restrict__ Cm, int64_t ldbc,
+                                                       const float* __restrict__ dt_raw, int64_t lddt, const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dv,
+                                                       const float* __restrict__ proj, int64_t ldp, int x_off, int z_off,
+                                                       float* __restrict__ S, float* __restrict__ conv_state, OT* __restrict__ out) {
+  extern __shared__ float bc[];            // [SS_TC][2][NP]: B | C of the chunk's tokens, NP = LPC * 16
+  constexpr int NP = LPC * SS_NS, CPB = 256 / LPC;
+  const int b = blockIdx.y, tid = threadIdx.x;
+  const int ch = blockIdx.x * CPB + tid / LPC, sl = tid % LPC, n0 = sl * SS_NS;
+  const bool live = ch < c.inner;
+  const int N = c.state, q0 = q_indptr[b], q1 = q_indptr[b + 1];
+  const bool cont = pos0[b] > 0;
+  float A[SS_NS], st[SS_NS];
+  float* Srow = S + ((size_t)slot[b] * c.inner + (live ? ch : 0)) * N;
+#pragma unroll
+  for (int i = 0; i < SS_NS; i++) {
+    const bool ok = live && n0 + i < N;
+    A[i] = ok ? -expf(A_log[(size_t)ch * N + n0 + i]) : 0.f;
+    st[i] = ok && cont ? Srow[n0 + i] : 0.f;
+  }
+  const float dtb = live ? dt_bias[ch] : 0.f, dsk = live ? Dv[ch] : 0.f;
+  for (int tc = q0; tc < q1; tc += SS_TC) {
+    const int nt = min(SS_TC, q1 - tc);
+    __syncthreads();
+    for (int e = tid; e < nt * 2 * NP; e += 256) {
+      const int tt = e / (2 * NP), r = e % (2 * NP), which = r / NP, n = r % NP;
+      bc[e] = n < N ? (which ? Cm : Bm)[(size_t)(tc + tt) * ldbc + n] : 0.f;
+    }
+    float dtv[SS_TC], xv[SS_TC], zv[SS_TC];
+#pragma unroll
+    for (int tt = 0; tt < SS_TC; tt++) {
+      const bool ok = live && tt < nt;
+      dtv[tt] = ok ? dt_raw[(size_t)(tc + tt) * lddt + ch] : 0.f;
+      xv[tt] = ok ? xc[(size_t)(tc + tt) * c.inner + ch] : 0.f;
+      zv[tt] = ok ? proj[(size_t)(tc + tt) * ldp + z_off + ch] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int tt = 0; tt < SS_TC; tt++) {
+      if (tt < nt) {                        // (uniform over the workgroup)
+        const float dt = softplus_f32(dtv[tt] + dtb);
+        const float dx = dt * xv[tt];
+        const float* Bt = bc + (size_t)tt * 2 * NP + n0;
+        const float* Ct = Bt + NP;
+        float y = 0.f;
+#pragma unroll
+        for (int i = 0; i < SS_NS; i++) {
+          st[i] = fmaf(__expf(dt * A[i]), st[i], dx * Bt[i]);
+          y = fmaf(st[i], Ct[i], y);
+        }
+#pragma unroll
+        for (int off = 1; off < LPC; off <<= 1) y += __shfl_xor(y, off);
+        if (live && sl == 0) st_elem(out, (size_t)(tc + tt) * c.inner + ch, (y + dsk * xv[tt]) * silu_f32(zv[tt]));
+      }
+    }
+  }
+  if (!live) return;
+#pragma unroll
+  for (int i = 0; i < SS_NS; i++)
+    if (n0 + i < N) Srow[n0 + i] = st[i];
+  if (sl == 0 && c.taps > 1) {             // the convolution's state moves on: its last taps - 1 inputs
+    const int K1 = c.taps - 1, nn = q1 - q0;
+    float* cs = conv_state + (size_t)slot[b] * K1 * c.inner + ch;
+    float keep[SSM_MAX_TAPS];
+#pragma unroll
+    for (int i = 0; i < SSM_MAX_TAPS; i++) {
+      if (i < K1) {
+        const int src = nn - K1 + i;
+        keep[i] = src >= 0 ? proj[(size_t)(q0 + src) * ldp + x_off + ch] : (cont ? cs[(size_t)(nn + i) * c.inner] : 0.f);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < SSM_MAX_TAPS; i++)
+      if (i < K1) cs[(size_t)i * c.inner] = keep[i];
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// router: one wavefront per token; lane holds outputs lane, lane + 64, ... (E <= 64 * SR_RE)
+constexpr int SR_RE = 16;
+__global__ void __launch_bounds__(256) softmax_route_kernel(int T, int E, int top, float sum_eps, const float* __restrict__ logits,
+                                                            int64_t ldl, const float* __restrict__ corr, int32_t* __restrict__ idx,
+                                                            float* __restrict__ wts) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t >= T) return;
+  float s[SR_RE], ch[SR_RE];
+  float mx = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < SR_RE; i++) {
+    const int e = lane + i * 64;
+    s[i] = e < E ? logits[(size_t)t * ldl + e] : -INFINITY;
+    mx = fmaxf(mx, s[i]);
+  }
+  mx = wave_max(mx);
+  float den = 0.f;
+#pragma unroll
+  for (int i = 0; i < SR_RE; i++) {
+    s[i] = lane + i * 64 < E ? expf(s[i] - mx) : 0.f;
+    den += s[i];
+  }
+  den = wave_sum(den);
+#pragma unroll
+  for (int i = 0; i < SR_RE; i++) {
+    const int e = lane + i * 64;
+    s[i] = s[i] / den;
+    ch[i] = e < E ? s[i] + (corr ? corr[e] : 0.f) : -INFINITY;
+  }
+  float sum = 0.f;
+  for (int k = 0; k < top; k++) {
+    float bv = -INFINITY;
+    int be = 0x7fffffff;
+#pragma unroll
+    for (int i = 0; i < SR_RE; i++) {
+      const int e = lane + i * 64;
+      if (e < E && ch[i] > bv) {
+        bv = ch[i];
+        be = e;
+      }
+    }
+    for (int off = 32; off; off >>= 1) {
+      const float ov = __shfl_xor(bv, off);
+      const int oe = __shfl_xor(be, off);
+      if (oe != 0x7fffffff && (be == 0x7fffffff || ov > bv || (ov == bv && oe < be))) {
+        bv = ov;
+        be = oe;
+      }
+    }
+    float sv = 0.f;
+#pragma unroll
+    for (int i = 0; i < SR_RE; i++)
+      if (lane + i * 64 == be) {
+        sv = s[i];
+        ch[i] = -INFINITY;
+      }
+    sv = wave_sum(sv);                     // the chosen output's score (its owner's value, zeros elsewhere)
+    sum += sv;
+    if (lane == 0) {
+      idx[(size_t)t * top + k] = be;
+      wts[(size_t)t * top + k] = sv;
+    }
+  }
+  const float f = 1.0f / (sum + sum_eps);
+  __builtin_amdgcn_wave_barrier();
+  if (lane == 0)
+    for (int k = 0; k < top; k++) wts[(size_t)t * top + k] *= f;
+}
+
+}  // namespace
+
+extern "C" {
+
+int ktx_resid_norm(int T, int W, float* d_x, const ktx_resid_args* a, ktx_stream_t stream) {
+  KTX_REQUIRE(a && T >= 0 && W > 0 && d_x, "ktx_resid_norm: T >= 0, W > 0, x");
+  KTX_REQUIRE((size_t)W * 4 <= 150 * 1024, "ktx_resid_norm: a row must fit the LDS");
+  const bool adds = a->y || a->ey;
+  KTX_REQUIRE(!a->ey || (a->pair_pos && a->topk_idx && a->topk_w && a->top > 0 && a->h_in && dtype_ok(a->h_dtype)),
+              "ktx_resid_norm: the gathered term needs pair_pos, topk_idx, topk_w, top, h_in");
+  KTX_REQUIRE(!a->y_norm_w || a->y, "ktx_resid_norm: y_norm_w without y");
+  KTX_REQUIRE(!a->rows || !adds, "ktx_resid_norm: a row gather only without an addition");
+  KTX_REQUIRE(!a->norm_g || (a->out && dtype_ok(a->out_dtype)), "ktx_resid_norm: the norm needs its output");
+  KTX_REQUIRE(a->halo <= 0 || (a->norm_g && !a->rows && a->B > 0 && a->q_indptr && a->pos0 && a->slot && a->tok_req && a->conv_state &&
+                               a->out_dtype == KTX_SEQ_F32),
+              "ktx_resid_norm: halo rows need the batch's tensors, the state and an fp32 output");
+  if (T == 0 || (!adds && !a->norm_g)) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)W * 4;
+#define KTX_RN_GO(OT, HT)                                                                        \
+  do {                                                                                           \
+    KTX_HIP(ktx_set_max_lds((const void*)resid_norm_kernel<OT, HT>, 150 * 1024));                \
+    resid_norm_kernel<OT, HT><<<T, 256, lds, st>>>(W, d_x, *a);                                  \
+  } while (0)
+  const bool obf = a->norm_g && a->out_dtype == KTX_SEQ_BF16, hbf = a->ey && a->h_dtype == KTX_SEQ_BF16;
+  if (obf && hbf) KTX_RN_GO(bf16_t, bf16_t);
+  else if (obf) KTX_RN_GO(bf16_t, float);
+  else if (hbf) KTX_RN_GO(float, bf16_t);
+  else KTX_RN_GO(float, float);
+#undef KTX_RN_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_input_conv(int B, int T, int W, int taps, const float* d_hx, const float* d_w, const int32_t* d_q_indptr, const int32_t* d_slot,
+                   const int32_t* d_tok_req, float* d_conv_state, void* d_out, int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(B >= 0 && T >= 0 && W > 0 && taps >= 2 && d_hx && d_w && d_q_indptr && d_slot && d_tok_req && d_conv_state && d_out &&
+                  dtype_ok(out_dtype),
+              "ktx_input_conv: taps >= 2, pointers");
+  if (T == 0) return 0;
+  const dim3 grid(T, (W + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32)
+    input_conv_kernel<float><<<grid, 256, 0, st>>>(W, taps, d_hx, d_w, d_q_indptr, d_slot, d_tok_req, d_conv_state, (float*)d_out);
+  else
+    input_conv_kernel<bf16_t><<<grid, 256, 0, st>>>(W, taps, d_hx, d_w, d_q_indptr, d_slot, d_tok_req, d_conv_state, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_rows_mul_lookup(int T, int n, const float* d_a, int64_t lda, const void* d_table, int table_dtype, int64_t ldt, int col0,
+                        const int32_t* d_tokens, void* d_out, int out_dtype, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && n > 0 && d_a && d_table && d_tokens && d_out && dtype_ok(table_dtype) && dtype_ok(out_dtype) && col0 >= 0 &&
+                  col0 + n <= ldt && lda >= n,
+              "ktx_rows_mul_lookup: arguments");
+  if (T == 0) return 0;
+  const size_t total = (size_t)T * n;
+  const unsigned blocks = (unsigned)((total + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_ML_GO(TT, OT) \
+  rows_mul_lookup_kernel<TT, OT><<<blocks, 256, 0, st>>>(total, n, d_a, lda, (const TT*)d_table, ldt, col0, d_tokens, (OT*)d_out)
+  if (table_dtype == KTX_SEQ_F32) {
+    if (out_dtype == KTX_SEQ_F32) KTX_ML_GO(float, float);
+    else KTX_ML_GO(float, bf16_t);
+  } else {
+    if (out_dtype == KTX_SEQ_F32) KTX_ML_GO(bf16_t, float);
+    else KTX_ML_GO(bf16_t, bf16_t);
+  }
+#undef KTX_ML_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int swa_check(const ktx_swa_config* c, const char* who) {
+  KTX_REQUIRE(c && c->heads > 0 && c->kv_heads > 0 && c->heads % c->kv_heads == 0 && c->dim > 0 && c->vdim > 0 && c->page_size > 0 &&
+                  dtype_ok(c->cache_dtype),
+              std::string(who) + ": heads a multiple of kv_heads, positive sizes, a known cache type");
+  KTX_REQUIRE(c->rot_dims >= 0 && c->rot_dims % 2 == 0 && c->rot_dims <= c->dim, std::string(who) + ": rot_dims even and at most dim");
+  KTX_REQUIRE(!c->rot_values || c->vdim % 2 == 0, std::string(who) + ": rotated values need an even vdim");
+  return 0;
+}
+
+int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t ldp, int q_off, int k_off, int v_off,
+                 const double* d_inv_freq, const double* d_v_inv_freq, const int32_t* d_pos, const int32_t* d_cache_loc, void* d_kcache,
+                 void* d_vcache, float* d_q_out, float* d_vcs, ktx_stream_t stream) {
+  if (swa_check(cfg, "ktx_swa_prep")) return -1;
+  KTX_REQUIRE(T >= 0 && d_proj && d_pos && d_cache_loc && d_kcache && d_vcache && d_q_out, "ktx_swa_prep: null pointer");
+  KTX_REQUIRE(cfg->rot_dims == 0 || d_inv_freq, "ktx_swa_prep: rotation without frequencies");
+  KTX_REQUIRE(!cfg->rot_values || (d_v_inv_freq && d_vcs), "ktx_swa_prep: rotated values need their frequencies and the table");
+  if (T == 0) return 0;
+  const size_t lds = ((size_t)cfg->rot_dims + (cfg->rot_values ? cfg->vdim : 0) + 2) * 4;
+  KTX_REQUIRE(lds <= 60 * 1024, "ktx_swa_prep: the angle tables must fit the LDS");
+  hipStream_t st = (hipStream_t)stream;
+  if (cfg->cache_dtype == KTX_SEQ_F32)
+    swa_prep_kernel<float><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, q_off, k_off, v_off, d_inv_freq, d_v_inv_freq, d_pos, d_cache_loc,
+                                                (float*)d_kcache, (float*)d_vcache, d_q_out, d_vcs);
+  else
+    swa_prep_kernel<bf16_t><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, q_off, k_off, v_off, d_inv_freq, d_v_inv_freq, d_pos, d_cache_loc,
+                                                 (bf16_t*)d_kcache, (bf16_t*)d_vcache, d_q_out, d_vcs);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+static int swa_merge(const ktx_swa_config* cfg, int T, int nsplit, const float* d_scratch, const float* d_sink, const float* d_vcs,
+                     void* d_out, int out_dtype, hipStream_t st) {
+  const dim3 mg(T, cfg->heads);
+  if (out_dtype == KTX_SEQ_F32)
+    swa_merge_kernel<float><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, cfg->vdim, nsplit, cfg->rot_values, d_scratch, d_sink, d_vcs,
+                                                                 (float*)d_out);
+  else
+    swa_merge_kernel<bf16_t><<<mg, 256, (size_t)nsplit * 8, st>>>(T, cfg->heads, cfg->vdim, nsplit, cfg->rot_values, d_scratch, d_sink, d_vcs,
+                                                                  (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const void* d_kcache, const void* d_vcache,
+                    const int32_t* d_tok_req, const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices,
+                    const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (swa_check(cfg, "ktx_swa_forward")) return -1;
+  KTX_REQUIRE(T >= 0 && d_q && d_kcache && d_vcache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_out && dtype_ok(out_dtype),
+              "ktx_swa_forward: null pointer");
+  KTX_REQUIRE(!cfg->rot_values || d_vcs, "ktx_swa_forward: rotated values need the table of their angles");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_swa_forward: 1 <= nsplit <= 4096, scratch when > 1");
+  if (T == 0) return 0;
+  const int D = cfg->dim, V = cfg->vdim, HPG = cfg->heads / cfg->kv_heads;
+  KTX_REQUIRE(V <= 256 * SW_NACC, "ktx_swa_forward: vdim <= 8192");
+  const size_t budget = 96 * 1024;
+  int HG = std::min(HPG, std::max(1, 256 * SW_NACC / V));
+  int KTN = 64;
+  auto lds_of = [&](int hg, int ktn) {
+    return ((size_t)hg * D + (size_t)ktn * (D + 1) + (size_t)ktn * (V + 1) + (size_t)hg * ktn + 3 * (size_t)hg + ktn) * 4;
+  };
+  while (KTN > 8 && lds_of(1, KTN) > budget) KTN /= 2;
+  while (HG > 1 && lds_of(HG, KTN) > budget) HG = (HG + 1) / 2;
+  KTX_REQUIRE(lds_of(HG, KTN) <= 150 * 1024, "ktx_swa_forward: one head's query and 8 keys and values do not fit the LDS");
+  const size_t lds = lds_of(HG, KTN);
+  const int parts = (HPG + HG - 1) / HG;
+  const dim3 grid(T, cfg->kv_heads * parts, nsplit);
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_SW_GO(KT, OT)                                                                                                          \
+  do {                                                                                                                             \
+    KTX_HIP(ktx_set_max_lds((const void*)swa_fwd_kernel<KT, OT>, 150 * 1024));                                                     \
+    swa_fwd_kernel<KT, OT><<<grid, 256, lds, st>>>(*cfg, T, HG, parts, KTN, d_q, (const KT*)d_kcache, (const KT*)d_vcache, d_tok_req, \
+                                                   d_pos, d_page_indptr, d_page_indices, d_sink, d_vcs, nsplit, d_scratch, (OT*)d_out); \
+  } while (0)
+  if (cfg->cache_dtype == KTX_SEQ_F32) {
+    if (out_dtype == KTX_SEQ_F32) KTX_SW_GO(float, float);
+    else KTX_SW_GO(float, bf16_t);
+  } else {
+    if (out_dtype == KTX_SEQ_F32) KTX_SW_GO(bf16_t, float);
+    else KTX_SW_GO(bf16_t, bf16_t);
+  }
+#undef KTX_SW_GO
+  KTX_HIP(hipGetLastError());
+  if (nsplit > 1) return swa_merge(cfg, T, nsplit, d_scratch, d_sink, d_vcs, d_out, out_dtype, st);
+  return 0;
+}
+
+int ktx_swa_mfma_eligible(const ktx_swa_config* c) {
+  if (!c || c->cache_dtype != KTX_SEQ_BF16) return 0;
+  if (c->dim % 32 != 0 || c->dim > 32 * SM_KSMAX) return 0;
+  const int V = c->vdim;
+  if (!(V == 32 || V == 64 || V == 96 || V == 128 || V == 256)) return 0;
+  return swa_mfma_lds(*c) <= 150 * 1024;
+}
+
+int ktx_swa_mfma(const ktx_swa_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache, const void* d_vcache,
+                 const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,
+                 const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (swa_check(cfg, "ktx_swa_mfma")) return -1;
+  KTX_REQUIRE(ktx_swa_mfma_eligible(cfg), "ktx_swa_mfma: bf16 caches, dim a multiple of 32 up to 256, vdim 32 / 64 / 96 / 128 / 256");
+  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_kcache && d_vcache && d_q_indptr && d_pos0 && d_page_indptr &&
+                  d_page_indices && d_out && dtype_ok(out_dtype),
+              "ktx_swa_mfma: null pointer");
+  KTX_REQUIRE(!cfg->rot_values || d_vcs, "ktx_swa_mfma: rotated values need the table of their angles");
+  KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_swa_mfma: 1 <= nsplit <= 4096, scratch when > 1");
+  KTX_REQUIRE(aligned16(d_q) && aligned16(d_kcache) && aligned16(d_vcache), "ktx_swa_mfma: 16-byte aligned q and caches");
+  if (B == 0 || T == 0 || max_q_len == 0) return 0;
+  const int HPG = cfg->heads / cfg->kv_heads;
+  const int row_tiles = (int)(((int64_t)max_q_len * HPG + 63) / 64);
+  KTX_REQUIRE(cfg->kv_heads <= 65535, "ktx_swa_mfma: up to 65535 key heads");
+  const dim3 grid((unsigned)B * row_tiles, cfg->kv_heads, nsplit);
+  const size_t lds = swa_mfma_lds(*cfg);
+  hipStream_t st = (hipStream_t)stream;
+  const int V = cfg->vdim;
+#define KTX_SM_GO(NT, OT)                                                                                                             \
+  do {                                                                                                                                \
+    KTX_HIP(ktx_set_max_lds((const void*)swa_mfma_kernel<NT, OT>, 150 * 1024));                                                       \
+    swa_mfma_kernel<NT, OT><<<grid, 256, lds, st>>>(*cfg, T, row_tiles, d_q, (const bf16_t*)d_kcache, (const bf16_t*)d_vcache,        \
+                                                    d_q_indptr, d_pos0, d_page_indptr, d_page_indices, d_sink, d_vcs, nsplit, d_scratch, \
+                                                    (OT*)d_out);                                                                      \
+  } while (0)
+#define KTX_SM_NT(OT)                  \
+  do {                                 \
+    if (V == 32) KTX_SM_GO(2, OT);     \
+    else if (V == 64) KTX_SM_GO(4, OT); \
+    else if (V == 96) KTX_SM_GO(6, OT); \
+    else if (V == 128) KTX_SM_GO(8, OT); \
+    else KTX_SM_GO(16, OT);            \
+  } while (0)
+  if (out_dtype == KTX_SEQ_F32) KTX_SM_NT(float);
+  else KTX_SM_NT(bf16_t);
+#undef KTX_SM_NT
+#undef KTX_SM_GO
+  KTX_HIP(hipGetLastError());
+  if (nsplit > 1) return swa_merge(cfg, T, nsplit, d_scratch, d_sink, d_vcs, d_out, out_dtype, st);
+  return 0;
+}
+
+static int ssm_check(const ktx_ssm_config* c, const char* who) {
+  KTX_REQUIRE(c && c->inner > 0 && c->state > 0 && c->state <= 256 && c->dt_rank > 0 && c->taps >= 1 && c->taps <= SSM_MAX_TAPS + 1,
+              std::string(who) + ": inner, dt_rank > 0, 0 < state <= 256, 1 <= taps <= 9");
+  return 0;
+}
+
+int ktx_ssm_conv(const ktx_ssm_config* cfg, int B, int T, const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_slot,
+                 const int32_t* d_tok_req, const float* d_proj, int64_t ldp, int x_off, const float* d_w, const float* d_bias,
+                 const float* d_conv_state, float* d_xc, ktx_stream_t stream) {
+  if (ssm_check(cfg, "ktx_ssm_conv")) return -1;
+  KTX_REQUIRE(B >= 0 && T >= 0 && d_q_indptr && d_pos0 && d_slot && d_tok_req && d_proj && d_w && d_xc && (cfg->taps == 1 || d_conv_state),
+              "ktx_ssm_conv: null pointer");
+  if (T == 0) return 0;
+  const dim3 grid(T, (cfg->inner + 255) / 256);
+  ssm_conv_kernel<<<grid, 256, 0, (hipStream_t)stream>>>(*cfg, d_q_indptr, d_pos0, d_slot, d_tok_req, d_proj, ldp, x_off, d_w, d_bias,
+                                                         d_conv_state, d_xc);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_ssm_scan(const ktx_ssm_config* cfg, int B, int T, int max_q_len, const int32_t* d_q_indptr, const int32_t* d_pos0,
+                 const int32_t* d_slot, const float* d_xc, const float* d_Bm, const float* d_Cm, int64_t ldbc, const float* d_dt_raw,
+                 int64_t lddt, const float* d_dt_bias, const float* d_A_log, const float* d_D, const float* d_proj, int64_t ldp, int x_off,
+                 int z_off, float* d_S, float* d_conv_state, void* d_out, int out_dtype, ktx_stream_t stream) {
+  if (ssm_check(cfg, "ktx_ssm_scan")) return -1;
+  KTX_REQUIRE(B >= 0 && T >= 0 && d_q_indptr && d_pos0 && d_slot && d_xc && d_Bm && d_Cm && d_dt_raw && d_dt_bias && d_A_log && d_D &&
+                  d_proj && d_S && d_out && dtype_ok(out_dtype) && (cfg->taps == 1 || d_conv_state),
+              "ktx_ssm_scan: null pointer");
+  KTX_REQUIRE(B <= 65535, "ktx_ssm_scan: up to 65535 requests");
+  if (B == 0 || T == 0) return 0;
+  (void)max_q_len;
+  int lpc = 1;
+  while (lpc * SS_NS < cfg->state) lpc *= 2;
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_SS_GO(LPC, OT)                                                                                                         \
+  do {                                                                                                                             \
+    const dim3 grid((cfg->inner + 256 / LPC - 1) / (256 / LPC), B);                                                                \
+    ssm_scan_kernel<LPC, OT><<<grid, 256, (size_t)SS_TC * 2 * LPC * SS_NS * 4, st>>>(                                              \
+        *cfg, d_q_indptr, d_pos0, d_slot, d_xc, d_Bm, d_Cm, ldbc, d_dt_raw, lddt, d_dt_bias, d_A_log, d_D, d_proj, ldp, x_off, z_off, \
+        d_S, d_conv_state, (OT*)d_out);                                                                                            \
+  } while (0)
+#define KTX_SS_LPC(OT)                  \
+  do {                                  \
+    if (lpc == 1) KTX_SS_GO(1, OT);     \
+    else if (lpc == 2) KTX_SS_GO(2, OT); \
+    else if (lpc == 4) KTX_SS_GO(4, OT); \
+    else if (lpc == 8) KTX_SS_GO(8, OT); \
+    else KTX_SS_GO(16, OT);             \
+  } while (0)
+  if (out_dtype == KTX_SEQ_F32) KTX_SS_LPC(float);
+  else KTX_SS_LPC(bf16_t);
+#undef KTX_SS_LPC
+#undef KTX_SS_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_softmax_route(int T, int E, int top, float sum_eps, const float* d_logits, int64_t ldl, const float* d_correction,
+                      int32_t* d_topk_idx, float* d_topk_w, ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && E > 0 && top > 0 && top <= E && E <= 64 * SR_RE && d_logits && d_topk_idx && d_topk_w && ldl >= E,
+              "ktx_softmax_route: 0 < top <= outputs <= 1024");
+  if (T == 0) return 0;
+  softmax_route_kernel<<<(T + 3) / 4, 256, 0, (hipStream_t)stream>>>(T, E, top, sum_eps, d_logits, ldl, d_correction, d_topk_idx, d_topk_w);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+}  // extern "C"

@@ -67,6 +67,17 @@ def _pilavik_cache(config, max_tokens, max_requests, dtype, device):
     return KHybridCache(pilavik_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
 
 
+def _sadosun_config(d, dtype):
+    from ktransformers_amd.models.modeling_sadosun import make_sadosun_config
+    return make_sadosun_config(d, dtype)
+
+
+def _sadosun_cache(config, max_tokens, max_requests, dtype, device):
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    from ktransformers_amd.models.modeling_sadosun import sadosun_layer_specs
+    return KHybridCache(sadosun_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
+
+
 def _cls(module: str, name: str):
     def get():
         import importlib
@@ -85,6 +96,8 @@ MODEL_REGISTRY = {
                           _mitotar_cache, dtypes=(torch.bfloat16, torch.float32)),
     "Pilavik": ModelEntry(_pilavik_config, _cls("ktransformers_amd.models.modeling_pilavik", "PilavikForCausalLM"), "Pilavik.yaml",
                           _pilavik_cache, dtypes=(torch.bfloat16, torch.float32)),
+    "Sadosun": ModelEntry(_sadosun_config, _cls("ktransformers_amd.models.modeling_sadosun", "SadosunForCausalLM"), "Sadosun.yaml",
+                          _sadosun_cache, dtypes=(torch.bfloat16, torch.float32)),
 }
 
 

@@ -174,9 +174,14 @@ class KHybridCache:
                                  un-normed keys, plus fp32 1 / rms(k) per row and key head;
       "latent": width          — a paged cache of latent rows [pages * page_size, width] (bf16 or fp32): what a latent attention keeps
                                  per token (normed latent + rotated key part);
+      "kv": (kv_heads, dim, vdim) — paged KEY rows [pages * page_size, kv_heads, dim] and VALUE rows [.., kv_heads, vdim] (bf16 or
+                                 fp32) for grouped-query attention, stored as the attention reads them (rotated, normed);
       "rec": (heads, dim, vdim)   — fp32 state slots S [slots, heads, dim, vdim], n [slots, heads, dim], m [slots, heads] (mLSTM);
       "delta": (heads, dim, vdim) — fp32 state slots S alone (delta rule);
-      "conv": (channels, taps)    — fp32 slots [slots, taps - 1, channels]: the inputs a short causal convolution still needs.
+      "ssm": (channels, state)    — fp32 state slots S [slots, channels, state] (selective scan);
+      "conv": (channels, taps)    — fp32 slots [slots, taps - 1, channels]: the inputs a short causal convolution still needs;
+      "pre": [(channels, taps), ...] — the same kind of slots for convolutions on what the layer's sublayers read, one per sublayer
+                                 (an entry with taps <= 1 or None holds nothing).
     A layer that runs several times with the same weights (a repeated block) has one spec, and so one cache or state, per run.
     A request holds a list of pages (grown as it grows) and one slot from admit() to release(); freed pages and slots go back on
     LIFO free lists and are handed out again without being cleared: the attention kernels never read past a request's length and
@@ -195,17 +200,27 @@ class KHybridCache:
         self.max_cache_len = self.num_pages * self.page_size
         rows = self.num_pages * self.page_size
         self.k_caches, self.k_inv, self.S, self.n, self.m, self.lat_caches, self.conv = [], [], [], [], [], [], []
+        self.v_caches, self.pre_conv = [], []
         for spec in self.layer_specs:
             a, r, lat, dl, cv = spec.get("attn"), spec.get("rec"), spec.get("latent"), spec.get("delta"), spec.get("conv")
-            if r and dl:
-                raise ValueError("KHybridCache: a layer run has one recurrent state (\"rec\" or \"delta\")")
+            kv, ssm = spec.get("kv"), spec.get("ssm")
+            if sum(1 for s_ in (r, dl, ssm) if s_) > 1:
+                raise ValueError("KHybridCache: a layer run has one recurrent state (\"rec\", \"delta\" or \"ssm\")")
+            if a and kv:
+                raise ValueError("KHybridCache: a layer run has one key cache (\"attn\" or \"kv\")")
+            self.v_caches.append(torch.zeros((rows, kv[0], kv[2]), dtype=dtype, device=self.device) if kv else None)
+            self.pre_conv.append([torch.zeros((self.max_requests, pc[1] - 1, pc[0]), dtype=torch.float32, device=self.device)
+                                  if pc and pc[1] > 1 else None for pc in (spec.get("pre") or [])])
+            if kv:
+                a = (kv[0], kv[1])
             self.k_caches.append(torch.zeros((rows, a[0], a[1]), dtype=dtype, device=self.device) if a else None)
+            a = spec.get("attn")
             self.k_inv.append(torch.zeros((rows, a[0]), dtype=torch.float32, device=self.device) if a else None)
             self.lat_caches.append(torch.zeros((rows, int(lat)), dtype=dtype, device=self.device) if lat else None)
             self.conv.append(torch.zeros((self.max_requests, cv[1] - 1, cv[0]), dtype=torch.float32, device=self.device)
                              if cv and cv[1] > 1 else None)
-            r = r or dl
-            self.S.append(torch.zeros((self.max_requests, r[0], r[1], r[2]), dtype=torch.float32, device=self.device) if r else None)
+            r = r or dl or ssm
+            self.S.append(torch.zeros((self.max_requests,) + tuple(r), dtype=torch.float32, device=self.device) if r else None)
             r = spec.get("rec")
             self.n.append(torch.zeros((self.max_requests, r[0], r[1]), dtype=torch.float32, device=self.device) if r else None)
             self.m.append(torch.zeros((self.max_requests, r[0]), dtype=torch.float32, device=self.device) if r else None)
@@ -232,7 +247,8 @@ class KHybridCache:
 
     def state_tensors(self) -> list:
         """Every per-slot tensor a step advances in place (what a caller saves around runs that must not count)."""
-        return [t for group in (self.S, self.n, self.m, self.conv) for t in group if t is not None]
+        return [t for group in (self.S, self.n, self.m, self.conv) for t in group if t is not None] + \
+            [t for group in self.pre_conv for t in group if t is not None]
 
     def live_tokens(self) -> int:
         return sum(r["len"] for r in self.requests.values())
@@ -251,6 +267,7 @@ class KHybridCache:
         grow = lambda t: None if t is None else torch.cat([t, torch.zeros((extra,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
         self.S, self.n, self.m = [grow(t) for t in self.S], [grow(t) for t in self.n], [grow(t) for t in self.m]
         self.conv = [grow(t) for t in self.conv]
+        self.pre_conv = [[grow(t) for t in group] for group in self.pre_conv]
         self.free_slots.extend(range(self.max_requests + extra - 1, self.max_requests - 1, -1))
         self.max_requests += extra
         self.generation += 1
@@ -260,6 +277,7 @@ class KHybridCache:
         grow = lambda t: None if t is None else torch.cat([t, torch.zeros((rows,) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)])
         self.k_caches, self.k_inv = [grow(t) for t in self.k_caches], [grow(t) for t in self.k_inv]
         self.lat_caches = [grow(t) for t in self.lat_caches]
+        self.v_caches = [grow(t) for t in self.v_caches]
         self.free_pages.extend(range(self.num_pages + extra - 1, self.num_pages - 1, -1))
         self.num_pages += extra
         self.max_cache_len = self.num_pages * self.page_size

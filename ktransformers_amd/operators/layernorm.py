@@ -101,3 +101,44 @@ class KLayerNormBias(BaseInjectedModule):
         nn_ = None if next_norm is None else (next_norm.weight_f32, next_norm.bias_f32, next_norm.eps, next_norm.compute_dtype or torch.float32)
         return gated_norm_add(x, self.weight_f32, self.bias_f32, self.eps, y=y, ybias=ybias, gate_logits=gate_logits, gate_bias=gate_bias,
                               expert_rows=expert_rows, pair_pos=pair_pos, topk_w=topk_w, next_norm=nn_)
+
+
+class KScalarRMSNorm(BaseInjectedModule):
+    """RMS norm whose weight is ONE number for all coordinates, over an fp32 residual stream: x * g / sqrt(mean(x^2) + eps).  It is
+    also the place where what the sublayers before it produced joins the residual: one launch (include/ktx_swa.h `ktx_resid_norm`)
+    adds a sublayer's output (optionally unit-RMS-normed with a weight vector first) and a mixture's weighted expert rows to x, norms
+    the updated rows and — when a causal input convolution follows (`conv=`, operators/conv.py KInputConv) — lays them out with each
+    request's convolution state in front, which `ktx_input_conv` then turns into what the sublayer reads.  `rows=` gathers rows (the
+    model's last norm).  Checkpoint tensor: the module's key (a 0-d or 1-element tensor)."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "eps", float(orig_module.eps))
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", None))
+        object.__setattr__(self, "g", None)
+
+    def load(self):
+        import torch
+        g = self.gguf_loader.load_tensor(self.key, device=torch.device(self.device)).to(torch.float32).reshape(-1).contiguous()
+        if g.numel() != 1:
+            raise ValueError(f"{self.key}: a scalar-weight norm takes one number, got {g.numel()}")
+        object.__setattr__(self, "g", g)
+
+    def forward(self, x, batch=None, conv=None, conv_state=None, y=None, y_norm=None, moe=None, rows=None, out_dtype=None):
+        """x fp32 [T, W] (+= y, moe, in place) -> the normed rows (through `conv` when given) in out_dtype."""
+        import torch
+        from ktransformers_amd._native_swa import input_conv, resid_norm
+        dt = out_dtype or self.compute_dtype or torch.float32
+        if conv is None or conv.taps <= 1:
+            return resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), rows=rows, out_dtype=dt)
+        hx = resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), halo=(conv.taps - 1, batch, conv_state))
+        return input_conv(hx, conv.weight_f32, batch, conv_state, out_dtype=dt)
+
+
+def residual_add(x, y=None, y_norm=None, moe=None):
+    """x fp32 [T, W] += y (unit-RMS-normed with y_norm = (weight, eps) first when given) + a mixture's weighted expert rows, in place
+    (`ktx_resid_norm` without its norm)."""
+    from ktransformers_amd._native_swa import resid_norm
+    if y is not None or moe is not None:
+        resid_norm(x, y=y, y_norm=y_norm, moe=moe)
+    return x
