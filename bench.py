@@ -1854,6 +1854,64 @@ class HybKernelTimer(SeqKernelTimer):
             setattr(mod, name, fn)
 
 
+def family_measure(args, dev, cfg, loader, timer_cls, window, T, ctx):
+    """Prefill (one prompt of T tokens) and decode (batch 1 and 8 at a context of ctx tokens) of one fp32-residual family through
+    load_model / BatchEngine, with a per-kernel table from `timer_cls`.  window: keys a token sees at most (0: all)."""
+    import contextlib
+    import io
+    from ktransformers_amd.models import load_model
+    from ktransformers_amd.util.batch_engine import BatchEngine
+
+    def timed_ms(fn, reps):
+        fn()
+        torch.cuda.synchronize(dev)
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            torch.cuda.synchronize(dev)
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return sorted(ts)[len(ts) // 2]
+
+    with contextlib.redirect_stdout(io.StringIO()):
+        model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=loader)
+    cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
+    eng = BatchEngine(model, cache, use_graph=not args.no_graph)
+    g = torch.Generator().manual_seed(5)
+    prompt = torch.randint(0, 32000, (T,), generator=g).tolist()
+    state = {"pairs": 0, "keys": 0}
+    seen = lambda n: min(n, window) if window else n
+
+    def prefill():
+        state.update(pairs=sum(seen(i + 1) for i in range(T)), keys=T)
+        eng.step([{"id": "p", "tokens": prompt, "want": [T - 1]}], ["p"])
+    ms = timed_ms(prefill, 3)
+    with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
+        prefill()
+    res = {"prefill": {"tok_s": round(T / ms * 1e3, 1), "ms": round(ms, 3), "per_kernel": kt.table(ms)}}
+    for B in (1, 8):
+        ids = [f"d{b}" for b in range(B)]
+        ctx_prompt = torch.randint(0, 32000, (ctx,), generator=g).tolist()
+        eng.step([{"id": r, "tokens": ctx_prompt, "want": []} for r in ids])
+
+        def decode():
+            n = seen(cache.seq_len(ids[0]))
+            state.update(pairs=B * n, keys=B * n)
+            eng.step([{"id": r, "tokens": [7], "want": [0]} for r in ids])
+        ms = timed_ms(decode, 20)
+        eng.use_graph = False           # the per-kernel pass brackets eager launches
+        with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
+            decode()
+        eng.use_graph = not args.no_graph
+        res[f"decode_bs{B}"] = {"tok_s": round(B / ms * 1e3, 1), "ms_per_step": round(ms, 3), "per_kernel": kt.table(ms),
+                                "graph": eng.use_graph}
+        for r in ids:
+            cache.release(r)
+    del model, cache, eng
+    torch.cuda.empty_cache()
+    return res
+
+
 def run_pilavik(args, dev):
     """Prefill (one prompt of --prefill-tokens) and decode (batch 1 and 8 at a 2048-token context) throughput of Pilavik at
     PILAVIK_SIZES, each beside Mitotar of equal width and depth, with a per-kernel table and the fraction of its roofline (bf16 MFMA
@@ -1869,55 +1927,7 @@ def run_pilavik(args, dev):
     record = {"metric": "pilavik_prefill_decode", "unit": "tok/s", "layers": n_layers, "prefill_tokens": T, "decode_ctx": ctx,
               "dtype": "bf16 weights / activations / latent cache, fp32 residual, scores, router, state", "data": "synthetic", "sizes": {}}
 
-    def timed_ms(fn, reps):
-        fn()
-        torch.cuda.synchronize(dev)
-        ts = []
-        for _ in range(reps):
-            t0 = time.perf_counter()
-            fn()
-            torch.cuda.synchronize(dev)
-            ts.append((time.perf_counter() - t0) * 1e3)
-        return sorted(ts)[len(ts) // 2]
-
-    def measure(cfg, loader, timer_cls, window):
-        with contextlib.redirect_stdout(io.StringIO()):
-            model, config, entry = load_model(cfg, dtype=torch.bfloat16, device=str(dev), loader=loader)
-        cache = entry.make_cache(config, 8 * (ctx + 64) + T, 16, torch.bfloat16, str(dev))
-        eng = BatchEngine(model, cache, use_graph=not args.no_graph)
-        g = torch.Generator().manual_seed(5)
-        prompt = torch.randint(0, 32000, (T,), generator=g).tolist()
-        state = {"pairs": 0, "keys": 0}
-        seen = lambda n: min(n, window) if window else n
-
-        def prefill():
-            state.update(pairs=sum(seen(i + 1) for i in range(T)), keys=T)
-            eng.step([{"id": "p", "tokens": prompt, "want": [T - 1]}], ["p"])
-        ms = timed_ms(prefill, 3)
-        with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
-            prefill()
-        res = {"prefill": {"tok_s": round(T / ms * 1e3, 1), "ms": round(ms, 3), "per_kernel": kt.table(ms)}}
-        for B in (1, 8):
-            ids = [f"d{b}" for b in range(B)]
-            ctx_prompt = torch.randint(0, 32000, (ctx,), generator=g).tolist()
-            eng.step([{"id": r, "tokens": ctx_prompt, "want": []} for r in ids])
-
-            def decode():
-                n = seen(cache.seq_len(ids[0]))
-                state.update(pairs=B * n, keys=B * n)
-                eng.step([{"id": r, "tokens": [7], "want": [0]} for r in ids])
-            ms = timed_ms(decode, 20)
-            eng.use_graph = False           # the per-kernel pass brackets eager launches
-            with timer_cls(lambda: (state["pairs"], state["keys"])) as kt:
-                decode()
-            eng.use_graph = not args.no_graph
-            res[f"decode_bs{B}"] = {"tok_s": round(B / ms * 1e3, 1), "ms_per_step": round(ms, 3), "per_kernel": kt.table(ms),
-                                    "graph": eng.use_graph}
-            for r in ids:
-                cache.release(r)
-        del model, cache, eng
-        torch.cuda.empty_cache()
-        return res
+    measure = lambda cfg, loader, timer_cls, window: family_measure(args, dev, cfg, loader, timer_cls, window, T, ctx)
 
     for name in sizes:
         sz = PILAVIK_SIZES[name]
@@ -1948,6 +1958,165 @@ def run_pilavik(args, dev):
                           "mitotar_prefill": v["mitotar"].get("prefill", {}).get("tok_s"),
                           "mitotar_decode_bs1": v["mitotar"].get("decode_bs1", {}).get("tok_s"),
                           "mitotar_decode_bs8": v["mitotar"].get("decode_bs8", {}).get("tok_s")}
+                      for k, v in record["sizes"].items()}}
+    print(json.dumps(line), flush=True)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# --sadosun: the grouped-query window-attention / selective-scan family with scalar norms, input convolutions, a softmax-routed mixture
+# with identity experts and per-layer token inputs (models/modeling_sadosun.py) at a few layer sizes, beside Pilavik — the closest
+# existing family: the same fp32 residual, cache manager, step function and graph replay, a sliding-window attention with a sink, a
+# recurrence behind short convolutions, a routed mixture — at equal width and depth
+# ---------------------------------------------------------------------------------------------------------------------
+SADOSUN_SIZES = {
+    # per block of 4 layers: attention, attention, scan, attention; every layer with a mixture feed-forward
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, vdim=128, window=1024, inner=2048, state=16, dt_rank=64, experts=16, identity=2,
+                  top=2, e_ff=704, side=64, pilavik="w1024"),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, inner=4096, state=16, dt_rank=128, experts=32,
+                  identity=4, top=4, e_ff=704, side=128, pilavik="w2048"),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, window=2048, inner=8192, state=16, dt_rank=256, experts=64,
+                  identity=4, top=6, e_ff=1024, side=256, pilavik="w4096"),
+}
+
+
+def sadosun_config(sz, n_layers, vocab=32000):
+    attn = {"type": "attention", "mixer": {"heads": sz["heads"], "kv_heads": sz["kv_heads"], "dim": sz["dim"], "vdim": sz["vdim"],
+                                           "scale": sz["dim"] ** -0.5, "mask": {"size": sz["window"]}, "rot": {"base": 10000.0, "dims": sz["dim"]}}}
+    scan = {"type": "mamba1", "mixer": {"inner": sz["inner"], "state": sz["state"], "dt_rank": sz["dt_rank"], "conv": 4}}
+    moe = {"kind": "moe", "expert": {"ff": sz["e_ff"]}, "router": {"experts": sz["experts"], "top": sz["top"], "identity": sz["identity"]}}
+    layers = [dict((attn, attn, scan, attn)[i % 4], mlp=moe) for i in range(n_layers)]
+    return {"architecture": "Sadosun", "width": sz["width"], "vocab": vocab, "norm": {"eps": 1e-5}, "embedding": {"scale": 8.0},
+            "canon": {"taps": 4}, "token_side": {"dim": sz["side"]}, "layers": layers}
+
+
+class SwaRandomLoader(HybRandomLoader):
+    """Random bf16 weights by tensor name for a Sadosun config (names and shapes of models/modeling_sadosun.py's checkpoint)."""
+
+    def __init__(self, cfg, dev):
+        self.dev, self.tensor_device_map, self.shapes = dev, {}, {}
+        W, S = cfg["width"], self.shapes
+        side, taps = (cfg.get("token_side") or {}).get("dim", 0), (cfg.get("canon") or {}).get("taps", 0)
+        S.update({"embed": (cfg["vocab"], W), "head": (cfg["vocab"], W), "final.norm": ()})
+        if side:
+            S["side.embed"] = (cfg["vocab"], side * len(cfg["layers"]))
+        for i, L in enumerate(cfg["layers"]):
+            p, m, c = f"l{i}.", L["mixer"], L.get("mlp")
+            for n in ("1",) + (("2",) if c else ()):
+                S[p + "norm" + n] = ()
+                if taps:
+                    S[p + "canon" + n] = (W, taps)
+            if L["type"] == "attention":
+                H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+                S.update({p + "mix.q": (H * D, W), p + "mix.k": (G * D, W), p + "mix.v": (G * V, W), p + "mix.o": (W, H * V)})
+            else:
+                I, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+                S.update({p + "mix.in": (2 * I, W), p + "mix.conv": (I, K), p + "mix.conv.b": (I,), p + "mix.x": (R + 2 * N, I),
+                          p + "mix.dt": (I, R), p + "mix.dt.b": (I,), p + "mix.A_log": (I, N), p + "mix.D": (I,), p + "mix.o": (W, I)})
+            if c:
+                F, r = c["expert"]["ff"], c["router"]
+                S[p + "mlp.router"] = (r["experts"] + r.get("identity", 0), W)
+                S[p + "mlp.correction"] = (r["experts"] + r.get("identity", 0),)
+                for e in range(r["experts"]):
+                    S.update({p + f"mlp.e{e}.up": (F, W), p + f"mlp.e{e}.down": (W, F)})
+            if side:
+                S.update({p + "side.gate": (side, W), p + "side.proj": (W, side), p + "side.norm": (W,)})
+
+    def load_tensor(self, name, device="cpu"):
+        import zlib
+        shape = self.shapes[name]
+        g = torch.Generator(device=self.dev)
+        g.manual_seed(zlib.crc32(name.encode()))
+        t = torch.randn(shape, generator=g, device=self.dev, dtype=torch.bfloat16)
+        leaf = name.rsplit(".", 1)[-1]
+        if leaf in ("norm1", "norm2", "norm") or name == "final.norm" or name.endswith(".D"):
+            return t.mul_(0.1).add_(1.0)
+        if name.endswith((".A_log", ".dt.b")):
+            return t.mul_(0.5).sub_(1.0)
+        if leaf in ("canon1", "canon2", "conv"):
+            return t.mul_(0.4)
+        if name.endswith((".conv.b", ".correction")):
+            return t.mul_(0.05)
+        if name in ("embed", "side.embed"):
+            return t
+        return t.mul_(shape[-1] ** -0.5)
+
+
+class SwaKernelTimer(HybKernelTimer):
+    """HIP events around every call of the window-attention / scan bindings and of the shared grouped and dense products."""
+    HYB = ("moe_plan", "expert_gemm")
+    SWA = ("resid_norm", "input_conv", "rows_mul_lookup", "swa_prep", "swa_forward", "swa_mfma", "ssm_conv", "ssm_scan", "softmax_route")
+
+    def _cost(self, name, a, kw, out):
+        nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0
+        if name in ("swa_forward", "swa_mfma"):
+            cfg, q, kc, vc = a[0], a[1], a[2], a[3]
+            pairs, keys = self.kv_len_of()
+            return name, 2.0 * pairs * cfg.heads * (cfg.dim + cfg.vdim), keys * cfg.kv_heads * (cfg.dim + cfg.vdim) * kc.element_size() + nb(q) + nb(out)
+        if name == "ssm_scan":
+            cfg, xc = a[0], a[1]
+            B = a[11].B
+            return name, 6.0 * xc.shape[0] * cfg.inner * cfg.state, 2.0 * B * cfg.inner * cfg.state * 4 + 3 * nb(xc) + nb(out)
+        if name == "resid_norm":
+            x = a[0]
+            n = 2 * nb(x) + nb(kw.get("y")) + nb(out)
+            if kw.get("moe") is not None:
+                n += kw["moe"][3].shape[1] * nb(x)
+            return name, 0.0, n
+        return super()._cost(name, a, kw, out)
+
+    def __enter__(self):
+        from ktransformers_amd import _native_hyb, _native_seq, _native_swa
+        for mod, names in ((_native_hyb, self.HYB), (_native_seq, self.SEQ), (_native_swa, self.SWA)):
+            for name in names:
+                fn = getattr(mod, name)
+                self.saved[(mod, name)] = fn
+
+                def wrapped(*a, _fn=fn, _name=name, **kw):
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    out = _fn(*a, **kw)
+                    e1.record()
+                    self.rows.append((e0, e1) + self._cost(_name, a, kw, out))
+                    return out
+                setattr(mod, name, wrapped)
+        return self
+
+
+def run_sadosun(args, dev):
+    """Prefill (one prompt of --prefill-tokens) and decode (batch 1 and 8 at a 2048-token context) throughput of Sadosun at
+    SADOSUN_SIZES, each beside Pilavik of equal width and depth, with a per-kernel table and the fraction of its roofline (bf16 MFMA
+    peak or HBM peak, whichever bounds).  Random weights, synthetic tokens.  Prints one JSON line; the whole record goes to
+    bench_sadosun.json beside this file."""
+    n_layers, T, ctx = args.layers or 4, args.prefill_tokens, 2048
+    sizes = [s for s in (args.sadosun.split(",") if args.sadosun != "all" else SADOSUN_SIZES) if s in SADOSUN_SIZES]
+    record = {"metric": "sadosun_prefill_decode", "unit": "tok/s", "layers": n_layers, "prefill_tokens": T, "decode_ctx": ctx,
+              "dtype": "bf16 weights / activations / key and value caches, fp32 residual, scores, router, state", "data": "synthetic",
+              "sizes": {}}
+    for name in sizes:
+        sz = SADOSUN_SIZES[name]
+        cfg = sadosun_config(sz, n_layers)
+        loader = SwaRandomLoader(cfg, dev)
+        res = family_measure(args, dev, cfg, loader, SwaKernelTimer, sz["window"], T, ctx)
+        active = loader.active_params(cfg) - math.prod(loader.shapes.get("side.embed", (0,)))
+        res["weights_GB"] = round(sum(math.prod(v) for k, v in loader.shapes.items() if k not in ("embed", "side.embed")) * 2 / 1e9, 3)
+        res["active_weights_GB"] = round(active * 2 / 1e9, 3)
+        res["decode_bs1"]["frac_of_hbm_peak"] = round(active * 2 / (res["decode_bs1"]["ms_per_step"] * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)
+        try:
+            psz = PILAVIK_SIZES[sz["pilavik"]]
+            pcfg = pilavik_config(psz, n_layers)
+            res["pilavik"] = family_measure(args, dev, pcfg, HybRandomLoader(pcfg, dev), HybKernelTimer, psz["window"], T, ctx)
+        except Exception as e:      # the comparison must not lose the new family's numbers
+            res["pilavik"] = {"error": f"{type(e).__name__}: {e}"}
+        record["sizes"][name] = res
+        log(f"[sadosun] {name}: prefill {res['prefill']['tok_s']} tok/s, decode bs1 {res['decode_bs1']['tok_s']} tok/s, "
+            f"bs8 {res['decode_bs8']['tok_s']} tok/s")
+    with open(os.path.join(ROOT, "bench_sadosun.json"), "w") as f:
+        json.dump(record, f, indent=1)
+    line = {"metric": record["metric"], "unit": "tok/s", "layers": n_layers, "data": "synthetic",
+            "sizes": {k: {"prefill": v["prefill"]["tok_s"], "decode_bs1": v["decode_bs1"]["tok_s"], "decode_bs8": v["decode_bs8"]["tok_s"],
+                          "pilavik_prefill": v["pilavik"].get("prefill", {}).get("tok_s"),
+                          "pilavik_decode_bs1": v["pilavik"].get("decode_bs1", {}).get("tok_s"),
+                          "pilavik_decode_bs8": v["pilavik"].get("decode_bs8", {}).get("tok_s")}
                       for k, v in record["sizes"].items()}}
     print(json.dumps(line), flush=True)
 
@@ -1995,6 +2164,11 @@ def main():
                     help="instead of the default workload: prefill / decode throughput of the Pilavik family (gated delta rule + latent "
                          "window attention, PolyNorm and mixture feed-forwards) at layer sizes from PILAVIK_SIZES (comma-separated, or "
                          "'all'), beside Mitotar of equal width and depth; one JSON line, detail in bench_pilavik.json")
+    ap.add_argument("--sadosun", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of the Sadosun family (grouped-query window "
+                         "attention with rotated values + selective scan, a softmax-routed mixture with identity experts) at layer sizes "
+                         "from SADOSUN_SIZES (comma-separated, or 'all'), beside Pilavik of equal width and depth; one JSON line, detail in "
+                         "bench_sadosun.json")
     ap.add_argument("--pmc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--trace-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -2020,6 +2194,10 @@ def main():
     if args.pilavik:
         torch.cuda.set_device(dev)
         run_pilavik(args, dev)
+        return
+    if args.sadosun:
+        torch.cuda.set_device(dev)
+        run_sadosun(args, dev)
         return
     torch.cuda.set_device(dev)
     if args.pmc_child:

@@ -122,7 +122,7 @@ def route(P, pre, c, h):
     correction per expert, the weights do not; weights are the chosen scores over their sum."""
     z = h @ P[pre + "router"].T
     s = torch.softmax(z, dim=-1)
-    choice = s + P[pre + "correction"]
+    choice = s + P[pre + "correction"] if pre + "correction" in P else s
     idx = torch.topk(choice, c["router"]["top"], dim=-1).indices
     w = torch.gather(s, 1, idx)
     return idx, w / (w.sum(dim=-1, keepdim=True) + ROUTER_SUM_EPS)
@@ -180,3 +180,81 @@ def forward(P, cfg, tokens, dtype=torch.float64, return_layers=False):
         trail.append(x.clone())
     logits = scalar_norm(x, P["final.norm"], eps) @ P["head"].T
     return (logits, torch.stack(trail)) if return_layers else logits
+
+
+# ---- small configurations and random checkpoints for the tests ---------------------------------------------------------------------
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, window=12, rot_dims=None, base=10000.0, scale=None, rot=True, mlp=None):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else dim ** -0.5}
+    if rot:
+        m["rot"] = {"base": base, "dims": dim if rot_dims is None else rot_dims}
+    if window:
+        m["mask"] = {"size": window}
+    return {"type": "attention", "mixer": m, "mlp": mlp}
+
+
+def scan_layer(inner=48, state=8, dt_rank=4, conv=3, mlp=None):
+    return {"type": "mamba1", "mixer": {"inner": inner, "state": state, "dt_rank": dt_rank, "conv": conv}, "mlp": mlp}
+
+
+def moe_mlp(experts=5, top=2, identity=2, ff=24):
+    return {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top, "identity": identity}}
+
+
+def make_config(layers, width=32, vocab=61, eps=1e-5, taps=3, side=6, scale=4.0):
+    cfg = {"architecture": "Sadosun", "width": width, "vocab": vocab, "norm": {"eps": eps}, "embedding": {"scale": scale}, "layers": layers}
+    if taps:
+        cfg["canon"] = {"taps": taps}
+    if side:
+        cfg["token_side"] = {"dim": side}
+    return cfg
+
+
+def random_checkpoint(cfg: dict, seed: int = 0) -> dict:
+    """Random bf16-representable weights with the checkpoint's tensor names for a config of the design."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def mat(o, i, s=None):
+        return (torch.randn(o, i, generator=g) * (s if s is not None else 1.0 / math.sqrt(i))).to(torch.bfloat16)
+
+    def vec(n, mean=0.0, s=0.1):
+        return (mean + torch.randn(n, generator=g) * s).to(torch.bfloat16)
+
+    def one(mean=1.0, s=0.2):
+        return (mean + torch.randn((), generator=g) * s).to(torch.bfloat16)
+
+    taps = (cfg.get("canon") or {}).get("taps")
+    side = (cfg.get("token_side") or {}).get("dim")
+    P = {"embed": mat(cfg["vocab"], W, 1.0), "head": mat(cfg["vocab"], W), "final.norm": one()}
+    if side:
+        P["side.embed"] = mat(cfg["vocab"], side * len(cfg["layers"]), 1.0)
+    for li, layer in enumerate(cfg["layers"]):
+        p, m = f"l{li}.", layer["mixer"]
+        P[p + "norm1"] = one()
+        if taps:
+            P[p + "canon1"] = mat(W, taps, 0.4)
+        if layer["type"] == "attention":
+            H, G, D, V = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
+            P[p + "mix.q"], P[p + "mix.k"], P[p + "mix.v"] = mat(H * D, W), mat(G * D, W), mat(G * V, W)
+            P[p + "mix.o"] = mat(W, H * V)
+        else:
+            I, N, R, K = m["inner"], m["state"], m["dt_rank"], m["conv"]
+            P[p + "mix.in"], P[p + "mix.conv"], P[p + "mix.conv.b"] = mat(2 * I, W), mat(I, K, 0.5), vec(I)
+            P[p + "mix.x"], P[p + "mix.dt"], P[p + "mix.dt.b"] = mat(R + 2 * N, I), mat(I, R), vec(I, -1.0, 1.0)
+            P[p + "mix.A_log"], P[p + "mix.D"], P[p + "mix.o"] = mat(I, N, 0.7), vec(I, 1.0, 0.3), mat(W, I)
+        c = layer.get("mlp")
+        if c:
+            P[p + "norm2"] = one()
+            if taps:
+                P[p + "canon2"] = mat(W, taps, 0.4)
+            E, ID, F = c["router"]["experts"], c["router"].get("identity") or 0, c["expert"]["ff"]
+            P[p + "mlp.router"], P[p + "mlp.correction"] = mat(E + ID, W, 2.0 / math.sqrt(W)), vec(E + ID, 0.0, 0.05)
+            for e in range(E):
+                P[p + f"mlp.e{e}.up"], P[p + f"mlp.e{e}.down"] = mat(F, W), mat(W, F)
+        if side:
+            P[p + "side.gate"], P[p + "side.proj"], P[p + "side.norm"] = mat(side, W, 0.5 / math.sqrt(W)), mat(W, side), vec(W, 0.7, 0.2)
+    return P
+
+
+def as_double(P: dict) -> dict:
+    return {k: (v.double() if v.is_floating_point() else v) for k, v in P.items()}

@@ -14,7 +14,11 @@ PAIRS = [("ktx_moe_config", "_MoeConfig", "ktx_moe.h"), ("ktx_linear_config", "_
          ("ktx_mla_config", "_MlaConfig", "ktx_mla.h"), ("ktx_gemm_args", "_GemmArgs", "ktx_gemm.h"),
          ("ktx_attn_decode_args", "_AttnDecodeArgs", "ktx_attn.h"),
          # (the sequence-mixer structs are mirrored in ktransformers_amd/_native_seq.py)
-         ("ktx_sigattn_config", "_SigAttnConfig", "ktx_seq.h"), ("ktx_mlstm_config", "_MlstmConfig", "ktx_seq.h")]
+         ("ktx_sigattn_config", "_SigAttnConfig", "ktx_seq.h"), ("ktx_mlstm_config", "_MlstmConfig", "ktx_seq.h"),
+         # (ktransformers_amd/_native_hyb.py, _native_swa.py)
+         ("ktx_delta_config", "_DeltaConfig", "ktx_hyb.h"), ("ktx_latattn_config", "_LatAttnConfig", "ktx_hyb.h"),
+         ("ktx_resid_args", "_ResidArgs", "ktx_swa.h"), ("ktx_swa_config", "_SwaConfig", "ktx_swa.h"),
+         ("ktx_ssm_config", "_SsmConfig", "ktx_swa.h")]
 
 
 @pytest.fixture(scope="module")
@@ -23,11 +27,14 @@ def native():
         from ktransformers_amd import _native
     except ImportError as e:          # the library is built by __graft_entry__.build(); without it there is nothing to mirror
         pytest.skip(f"libktx_hip.so not built: {e}")
-    from ktransformers_amd import _native_seq
+    from ktransformers_amd import _native_hyb, _native_seq, _native_swa
 
     class Both:
         def __getattr__(self, name):
-            return getattr(_native, name) if hasattr(_native, name) else getattr(_native_seq, name)
+            for mod in (_native, _native_seq, _native_hyb, _native_swa):
+                if hasattr(mod, name):
+                    return getattr(mod, name)
+            raise AttributeError(name)
     return Both()
 
 
