@@ -42,7 +42,10 @@ typedef struct ktx_resid_args {
    * rows (int32 [T], optional, only without an addition): out[i] = norm(x[rows[i]]).
    * halo > 0 (requires B, q_indptr, pos0, slot, tok_req, conv_state): out is fp32 [T + B * halo][W]; request b's rows are preceded by
    * `halo` rows holding conv_state[slot[b]] (fp32 [slots][halo][W]; zeros when pos0[b] == 0): token t of request b is row
-   * t + (b + 1) * halo — the layout ktx_input_conv reads. */
+   * t + (b + 1) * halo — the layout ktx_input_conv reads.
+   * conv_w (fp32 [W][conv_taps], instead of halo; same batch tensors; EVERY request brings exactly one token; 2 <= conv_taps <= 9): the
+   * input convolution in the same launch — out[t] = h + conv(h) of out_dtype with h = the normed row and the slot's state before it,
+   * and the slot's state moves on by one token. */
   const float* norm_g;
   float eps;
   const int32_t* rows;
@@ -51,7 +54,9 @@ typedef struct ktx_resid_args {
   const int32_t* pos0;
   const int32_t* slot;
   const int32_t* tok_req;
-  const float* conv_state;
+  float* conv_state;
+  const float* conv_w;
+  int32_t conv_taps;
   void* out;
   int32_t out_dtype;
 } ktx_resid_args;
@@ -101,7 +106,7 @@ int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const vo
 
 /* The same operator on the matrix cores for prompts, portions and decode steps: the (token, head) pairs of a request that share a key
  * head are the rows of one query matrix; workgroups of 64 rows walk 32-key tiles, bf16 MFMA for q . k and weights x values, scores /
- * mask / softmax in fp32.  Eligible: bf16 caches, dim a multiple of 32 up to 256, vdim a multiple of 16 up to 256. */
+ * mask / softmax in fp32.  Eligible: bf16 caches, dim a multiple of 32 up to 256, vdim 32 / 64 / 96 / 128 / 256. */
 int ktx_swa_mfma_eligible(const ktx_swa_config* cfg);
 int ktx_swa_mfma(const ktx_swa_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache, const void* d_vcache,
                  const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,

@@ -16,8 +16,8 @@ _P, _I, _L, _F, _I32 = C.c_void_p, C.c_int, C.c_int64, C.c_float, C.c_int32
 class _ResidArgs(C.Structure):       # include/ktx_swa.h: ktx_resid_args
     _fields_ = [("y", _P), ("ldy", _L), ("y_norm_w", _P), ("y_norm_eps", _F), ("ey", _P), ("pair_pos", _P), ("topk_idx", _P), ("topk_w", _P),
                 ("top", _I32), ("n_real", _I32), ("h_in", _P), ("h_dtype", _I32), ("norm_g", _P), ("eps", _F), ("rows", _P), ("halo", _I32),
-                ("B", _I32), ("q_indptr", _P), ("pos0", _P), ("slot", _P), ("tok_req", _P), ("conv_state", _P), ("out", _P),
-                ("out_dtype", _I32)]
+                ("B", _I32), ("q_indptr", _P), ("pos0", _P), ("slot", _P), ("tok_req", _P), ("conv_state", _P), ("conv_w", _P),
+                ("conv_taps", _I32), ("out", _P), ("out_dtype", _I32)]
 
 
 class _SwaConfig(C.Structure):       # include/ktx_swa.h: ktx_swa_config
@@ -44,6 +44,9 @@ lib.ktx_ssm_scan.argtypes = [C.POINTER(_SsmConfig), _I, _I, _I, _P, _P, _P, _P, 
 lib.ktx_softmax_route.argtypes = [_I, _I, _I, _F, _P, _L, _P, _P, _P, _P]
 
 
+FUSED_CONV_MAX_TAPS = 9      # ktx_resid_norm's one-token form keeps the state rows of one channel in registers
+
+
 def _ptr(t):
     return t.data_ptr() if t is not None else None
 
@@ -66,12 +69,14 @@ def _rows_f32(t, what):
 
 
 def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | None = None, moe: tuple | None = None,
-               norm: tuple | None = None, halo: tuple | None = None, rows: torch.Tensor | None = None, out_dtype=torch.float32):
+               norm: tuple | None = None, halo: tuple | None = None, rows: torch.Tensor | None = None, out_dtype=torch.float32,
+               conv: tuple | None = None):
     """One launch (ktx_resid_norm): x [T, W] fp32 += y (with y_norm = (weight [W], eps): y / rms(y) * weight first)
     + the mixture's weighted sum, moe = (expert_rows [pairs, W], pair_pos, topk_idx, topk_w [T, top], n_real, h_in [T, W]); then, with
     norm = (g: one fp32 number on the device, eps), returns x * g / rms(x) — in out_dtype [T or len(rows), W], or, with
     halo = (taps - 1, batch, conv_state [slots, taps - 1, W]), as fp32 [T + B * halo, W] with every request's state rows in front of
-    its tokens (what input_conv reads)."""
+    its tokens (what input_conv reads).  conv = (taps weight fp32 [W, taps], batch, conv_state), for steps in which every request brings
+    exactly ONE token: h + conv(h) in out_dtype [T, W] from the same launch, the slots' state moved on."""
     _f32(x, "resid_norm x")
     T, W = x.shape
     a = _ResidArgs()
@@ -115,6 +120,17 @@ def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | N
                                                      batch.tok_req.data_ptr())
             a.conv_state = state.data_ptr()
             n_out = T + batch.B * h
+        if conv is not None:
+            cw, batch, state = conv
+            _f32(cw, "resid_norm conv weight"), _f32(state, "resid_norm conv_state")
+            taps = cw.shape[1]
+            if halo is not None or rows is not None or cw.shape[0] != W or not 2 <= taps <= FUSED_CONV_MAX_TAPS or batch.max_q_len != 1 or \
+                    batch.T != T or tuple(state.shape[1:]) != (taps - 1, W):
+                raise KtxError("resid_norm: the fused convolution takes one token per request, 2 .. 9 taps, a state [slots, taps - 1, W]")
+            a.conv_w, a.conv_taps, a.B = cw.data_ptr(), taps, int(batch.B)
+            a.q_indptr, a.pos0, a.slot, a.tok_req = (batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
+                                                     batch.tok_req.data_ptr())
+            a.conv_state = state.data_ptr()
         out = torch.empty((n_out, W), dtype=out_dtype, device=x.device)
         a.out, a.out_dtype = out.data_ptr(), SEQ_DTYPE[out_dtype]
     check(lib.ktx_resid_norm(rows.numel() if rows is not None else T, W, x.data_ptr(), C.byref(a), _stream_ptr(x.device)))

@@ -24,6 +24,7 @@ int dtype_ok(int d) { return d == KTX_SEQ_F32 || d == KTX_SEQ_BF16; }
 
 // ---------------------------------------------------------------------------------------------------------------------
 // one row per workgroup; the row lives in LDS between the passes
+constexpr int RN_MAX_HALO = 8, RN_TOP = 8;
 template <typename OT, typename HT>
 __global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restrict__ x, ktx_resid_args a) {
   extern __shared__ float row[];
@@ -45,15 +46,30 @@ __global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restric
       for (int e = tid; e < W; e += 256) row[e] = a.y_norm_w ? y[e] * r * a.y_norm_w[e] : y[e];
     }
     if (a.ey) {
+      // a step of one token is one workgroup: the choices' indices, weights and row numbers are fetched side by side, then the rows
+      // (a chain of dependent loads per choice would cost a memory round trip each)
       const HT* h = reinterpret_cast<const HT*>(a.h_in) + (size_t)t * W;
-      for (int k = 0; k < a.top; k++) {
-        const int g = a.topk_idx[(size_t)t * a.top + k];
-        const float w = a.topk_w[(size_t)t * a.top + k];
-        if (g < a.n_real) {
-          const float* src = a.ey + (size_t)a.pair_pos[(size_t)t * a.top + k] * W;
-          for (int e = tid; e < W; e += 256) row[e] += w * src[e];
-        } else {
-          for (int e = tid; e < W; e += 256) row[e] += w * ld_elem(h, e);
+      for (int k0 = 0; k0 < a.top; k0 += RN_TOP) {
+        int g[RN_TOP];
+        float w[RN_TOP];
+        const float* src[RN_TOP];
+#pragma unroll
+        for (int j = 0; j < RN_TOP; j++) {
+          const bool ok = k0 + j < a.top;
+          const size_t at = (size_t)t * a.top + (ok ? k0 + j : 0);
+          g[j] = ok ? a.topk_idx[at] : a.n_real;
+          w[j] = ok ? a.topk_w[at] : 0.f;
+          src[j] = a.ey + (size_t)a.pair_pos[at] * W;
+        }
+        for (int e = tid; e < W; e += 256) {
+          const float hv = ld_elem(h, e);
+          float v[RN_TOP];
+#pragma unroll
+          for (int j = 0; j < RN_TOP; j++) v[j] = g[j] < a.n_real ? src[j][e] : hv;
+          float acc = row[e];
+#pragma unroll
+          for (int j = 0; j < RN_TOP; j++) acc += w[j] * v[j];
+          row[e] = acc;
         }
       }
     }
@@ -70,6 +86,29 @@ __global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restric
   for (int e = tid; e < W; e += 256) s += row[e] * row[e];
   const float r = a.norm_g[0] / sqrtf(block_sum256(s, red) / (float)W + a.eps);
   OT* out = reinterpret_cast<OT*>(a.out);
+  if (a.conv_w) {                // one new token per request: the convolution and the state's move happen here
+    const int b = a.tok_req[t], taps = a.conv_taps, halo = taps - 1;
+    const bool cont = a.pos0[b] > 0;
+    float* st = a.conv_state + (size_t)a.slot[b] * halo * W;
+    for (int e = tid; e < W; e += 256) {
+      const float hn = row[e] * r;
+      float prev[RN_MAX_HALO];
+      float acc = 0.f;
+#pragma unroll
+      for (int j = 0; j < RN_MAX_HALO; j++) {
+        if (j < halo) {
+          prev[j] = cont ? st[(size_t)j * W + e] : 0.f;
+          acc += a.conv_w[(size_t)e * taps + j] * prev[j];
+        }
+      }
+      acc += a.conv_w[(size_t)e * taps + halo] * hn;
+      st_elem(out, (size_t)t * W + e, hn + acc);
+#pragma unroll
+      for (int j = 0; j < RN_MAX_HALO; j++)
+        if (j < halo) st[(size_t)j * W + e] = j + 1 < halo ? prev[(j + 1) % RN_MAX_HALO] : hn;
+    }
+    return;
+  }
   if (a.halo <= 0) {
     for (int e = tid; e < W; e += 256) st_elem(out, (size_t)i * W + e, row[e] * r);
     return;
@@ -566,9 +605,33 @@ __global__ void __launch_bounds__(256) ssm_conv_kernel(ktx_ssm_config c, const i
 }
 
 // The recurrence: a workgroup owns 256 / LPC channels of one request; a channel's state entries are split over LPC neighbouring lanes
-// (16 each, in registers).  Tokens are taken SS_TC at a time: the step's B and C rows of the chunk are staged in LDS once for all
-// channels, the per-channel inputs (step, x, gate) requested for the whole chunk before the sequential part starts.
-constexpr int SS_NS = 16, SS_TC = 8;
+// (SS_NS each, in registers), their read-outs joined with DPP inside the 16-lane row (lane shuffles beyond it).  Tokens are taken SS_TC
+// at a time: the chunk's B and C rows are staged in LDS once for all channels (two buffers, ONE barrier per chunk), the per-channel
+// inputs of the NEXT chunk (step, x, gate) and its B | C rows are requested before the sequential part of the current one starts, and
+// the steps' softplus, dt * x and the gate of a whole chunk are taken off the sequential path and shared by the lanes of a channel
+// (each takes a part of the chunk's tokens; the values reach the others by DPP when they are used).
+constexpr int SS_NS = 4, SS_TC = 16;
+template <int LPC>
+__device__ __forceinline__ float ssm_join(float y) {
+  if constexpr (LPC >= 2) y += ktx_dpp_f<KTX_DPP_QUAD_1032>(y);
+  if constexpr (LPC >= 4) y += ktx_dpp_f<KTX_DPP_QUAD_2301>(y);
+  if constexpr (LPC >= 8) y += ktx_dpp_f<KTX_DPP_ROW_HALF_MIRROR>(y);
+  if constexpr (LPC >= 16) y += ktx_dpp_f<KTX_DPP_ROW_MIRROR>(y);
+  if constexpr (LPC >= 32) y += __shfl_xor(y, 16);
+  if constexpr (LPC >= 64) y += __shfl_xor(y, 32);
+  return y;
+}
+
+// value v of lane k of the SH lanes that share a channel's per-token work (SH = 1, 2 or 4 neighbouring lanes inside a quad)
+template <int SH>
+__device__ __forceinline__ float ssm_bcast(float v, int k) {
+  if constexpr (SH == 1) return v;
+  else if constexpr (SH == 2) return k == 0 ? ktx_dpp_f<0xA0>(v) : ktx_dpp_f<0xF5>(v);          // quad_perm [0,0,2,2] / [1,1,3,3]
+  else return k == 0 ? ktx_dpp_f<0x00>(v) : k == 1 ? ktx_dpp_f<0x55>(v) : k == 2 ? ktx_dpp_f<0xAA>(v) : ktx_dpp_f<0xFF>(v);
+}
+// v_exp_f32 + v_rcp_f32, about 1 ulp each: the gate multiplies a read-out, it enters no recurrence
+__device__ __forceinline__ float silu_fast(float z) { return z * __builtin_amdgcn_rcpf(1.0f + __expf(-z)); }
+
 template <int LPC, typename OT>
 __global__ void __launch_bounds__(256) ssm_scan_kernel(ktx_ssm_config c, const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
                                                        const int32_t* __restrict__ slot, const float* __restrict__ xc,
@@ -577,10 +640,12 @@ __global__ void __launch_bounds__(256) ssm_scan_kernel(ktx_ssm_config c, const i
                                                        const float* __restrict__ A_log, const float* __restrict__ Dv,
                                                        const float* __restrict__ proj, int64_t ldp, int x_off, int z_off,
                                                        float* __restrict__ S, float* __restrict__ conv_state, OT* __restrict__ out) {
-  extern __shared__ float bc[];            // [SS_TC][2][NP]: B | C of the chunk's tokens, NP = LPC * 16
-  constexpr int NP = LPC * SS_NS, CPB = 256 / LPC;
+  constexpr int NP = LPC * SS_NS, CPB = 256 / LPC, CH = SS_TC * 2 * NP;     // CH floats of B | C per chunk
+  constexpr int PER = (CH + 255) / 256;                                      // of them per thread
+  constexpr int SH = LPC >= 4 ? 4 : LPC, MINE = SS_TC / SH;                  // lanes that share a channel's per-token work; tokens per lane
+  extern __shared__ __attribute__((aligned(16))) float bc[];                 // [2][SS_TC][2][NP]
   const int b = blockIdx.y, tid = threadIdx.x;
-  const int ch = blockIdx.x * CPB + tid / LPC, sl = tid % LPC, n0 = sl * SS_NS;
+  const int ch = blockIdx.x * CPB + tid / LPC, sl = tid % LPC, n0 = sl * SS_NS, sh = sl % SH;
   const bool live = ch < c.inner;
   const int N = c.state, q0 = q_indptr[b], q1 = q_indptr[b + 1];
   const bool cont = pos0[b] > 0;
@@ -593,40 +658,71 @@ __global__ void __launch_bounds__(256) ssm_scan_kernel(ktx_ssm_config c, const i
     st[i] = ok && cont ? Srow[n0 + i] : 0.f;
   }
   const float dtb = live ? dt_bias[ch] : 0.f, dsk = live ? Dv[ch] : 0.f;
-  for (int tc = q0; tc < q1; tc += SS_TC) {
+  // lane `sh` of a channel's sharing lanes takes the chunk's tokens sh, sh + SH, ...: their step, x and gate
+  float ndt[MINE], nx[MINE], nz[MINE], nbc[PER];
+  auto request = [&](int tc) {       // the chunk that starts at token tc: this lane's tokens and its share of the B | C rows
     const int nt = min(SS_TC, q1 - tc);
-    __syncthreads();
-    for (int e = tid; e < nt * 2 * NP; e += 256) {
-      const int tt = e / (2 * NP), r = e % (2 * NP), which = r / NP, n = r % NP;
-      bc[e] = n < N ? (which ? Cm : Bm)[(size_t)(tc + tt) * ldbc + n] : 0.f;
-    }
-    float dtv[SS_TC], xv[SS_TC], zv[SS_TC];
 #pragma unroll
-    for (int tt = 0; tt < SS_TC; tt++) {
+    for (int i = 0; i < MINE; i++) {
+      const int tt = i * SH + sh;
       const bool ok = live && tt < nt;
-      dtv[tt] = ok ? dt_raw[(size_t)(tc + tt) * lddt + ch] : 0.f;
-      xv[tt] = ok ? xc[(size_t)(tc + tt) * c.inner + ch] : 0.f;
-      zv[tt] = ok ? proj[(size_t)(tc + tt) * ldp + z_off + ch] : 0.f;
+      ndt[i] = ok ? dt_raw[(size_t)(tc + tt) * lddt + ch] : 0.f;
+      nx[i] = ok ? xc[(size_t)(tc + tt) * c.inner + ch] : 0.f;
+      nz[i] = ok ? proj[(size_t)(tc + tt) * ldp + z_off + ch] : 0.f;
     }
-    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+      const int e = tid + k * 256;
+      const int tt = e / (2 * NP), r = e % (2 * NP), which = r / NP, n = r % NP;
+      nbc[k] = e < CH && tt < nt && n < N ? (which ? Cm : Bm)[(size_t)(tc + tt) * ldbc + n] : 0.f;
+    }
+  };
+  auto stage = [&](int buf) {
+#pragma unroll
+    for (int k = 0; k < PER; k++) {
+      const int e = tid + k * 256;
+      if (e < CH) bc[buf * CH + e] = nbc[k];
+    }
+  };
+  if (q0 < q1) {
+    request(q0);
+    stage(0);
+  }
+  __syncthreads();
+  int buf = 0;
+  for (int tc = q0; tc < q1; tc += SS_TC, buf ^= 1) {
+    const int nt = min(SS_TC, q1 - tc);
+    float dt[MINE], dx[MINE], gz[MINE], sk[MINE];
+#pragma unroll
+    for (int i = 0; i < MINE; i++) {          // independent of the state: off the sequential path
+      dt[i] = softplus_f32(ndt[i] + dtb);
+      dx[i] = dt[i] * nx[i];
+      sk[i] = dsk * nx[i];
+      gz[i] = silu_fast(nz[i]);
+    }
+    const bool more = tc + SS_TC < q1;
+    if (more) request(tc + SS_TC);           // in flight while this chunk runs
+    const float* cur = bc + buf * CH;
 #pragma unroll
     for (int tt = 0; tt < SS_TC; tt++) {
       if (tt < nt) {                        // (uniform over the workgroup)
-        const float dt = softplus_f32(dtv[tt] + dtb);
-        const float dx = dt * xv[tt];
-        const float* Bt = bc + (size_t)tt * 2 * NP + n0;
-        const float* Ct = Bt + NP;
+        const float dtv = ssm_bcast<SH>(dt[tt / SH], tt % SH), dxv = ssm_bcast<SH>(dx[tt / SH], tt % SH);
+        const float skv = ssm_bcast<SH>(sk[tt / SH], tt % SH), gzv = ssm_bcast<SH>(gz[tt / SH], tt % SH);
+        const float4 Bt = *reinterpret_cast<const float4*>(cur + (size_t)tt * 2 * NP + n0);
+        const float4 Ct = *reinterpret_cast<const float4*>(cur + (size_t)tt * 2 * NP + NP + n0);
+        const float Bv[4] = {Bt.x, Bt.y, Bt.z, Bt.w}, Cv[4] = {Ct.x, Ct.y, Ct.z, Ct.w};
         float y = 0.f;
 #pragma unroll
         for (int i = 0; i < SS_NS; i++) {
-          st[i] = fmaf(__expf(dt * A[i]), st[i], dx * Bt[i]);
-          y = fmaf(st[i], Ct[i], y);
+          st[i] = fmaf(__expf(dtv * A[i]), st[i], dxv * Bv[i]);
+          y = fmaf(st[i], Cv[i], y);
         }
-#pragma unroll
-        for (int off = 1; off < LPC; off <<= 1) y += __shfl_xor(y, off);
-        if (live && sl == 0) st_elem(out, (size_t)(tc + tt) * c.inner + ch, (y + dsk * xv[tt]) * silu_f32(zv[tt]));
+        y = ssm_join<LPC>(y);
+        if (live && sl == 0) st_elem(out, (size_t)(tc + tt) * c.inner + ch, (y + skv) * gzv);
       }
     }
+    if (more) stage(buf ^ 1);
+    __syncthreads();
   }
   if (!live) return;
 #pragma unroll
@@ -735,6 +831,9 @@ int ktx_resid_norm(int T, int W, float* d_x, const ktx_resid_args* a, ktx_stream
   KTX_REQUIRE(a->halo <= 0 || (a->norm_g && !a->rows && a->B > 0 && a->q_indptr && a->pos0 && a->slot && a->tok_req && a->conv_state &&
                                a->out_dtype == KTX_SEQ_F32),
               "ktx_resid_norm: halo rows need the batch's tensors, the state and an fp32 output");
+  KTX_REQUIRE(!a->conv_w || (a->halo <= 0 && a->norm_g && !a->rows && a->conv_taps >= 2 && a->conv_taps <= RN_MAX_HALO + 1 && a->q_indptr &&
+                             a->pos0 && a->slot && a->tok_req && a->conv_state),
+              "ktx_resid_norm: the fused convolution needs 2 <= taps <= 9, the batch's tensors and the state, and no halo");
   if (T == 0 || (!adds && !a->norm_g)) return 0;
   hipStream_t st = (hipStream_t)stream;
   const size_t lds = (size_t)W * 4;
@@ -966,7 +1065,7 @@ int ktx_ssm_scan(const ktx_ssm_config* cfg, int B, int T, int max_q_len, const i
 #define KTX_SS_GO(LPC, OT)                                                                                                         \
   do {                                                                                                                             \
     const dim3 grid((cfg->inner + 256 / LPC - 1) / (256 / LPC), B);                                                                \
-    ssm_scan_kernel<LPC, OT><<<grid, 256, (size_t)SS_TC * 2 * LPC * SS_NS * 4, st>>>(                                              \
+    ssm_scan_kernel<LPC, OT><<<grid, 256, (size_t)2 * SS_TC * 2 * LPC * SS_NS * 4, st>>>(                                          \
         *cfg, d_q_indptr, d_pos0, d_slot, d_xc, d_Bm, d_Cm, ldbc, d_dt_raw, lddt, d_dt_bias, d_A_log, d_D, d_proj, ldp, x_off, z_off, \
         d_S, d_conv_state, (OT*)d_out);                                                                                            \
   } while (0)
@@ -976,7 +1075,9 @@ int ktx_ssm_scan(const ktx_ssm_config* cfg, int B, int T, int max_q_len, const i
     else if (lpc == 2) KTX_SS_GO(2, OT); \
     else if (lpc == 4) KTX_SS_GO(4, OT); \
     else if (lpc == 8) KTX_SS_GO(8, OT); \
-    else KTX_SS_GO(16, OT);             \
+    else if (lpc == 16) KTX_SS_GO(16, OT); \
+    else if (lpc == 32) KTX_SS_GO(32, OT); \
+    else KTX_SS_GO(64, OT);             \
   } while (0)
   if (out_dtype == KTX_SEQ_F32) KTX_SS_LPC(float);
   else KTX_SS_LPC(bf16_t);

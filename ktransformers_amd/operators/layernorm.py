@@ -108,8 +108,8 @@ class KScalarRMSNorm(BaseInjectedModule):
     also the place where what the sublayers before it produced joins the residual: one launch (include/ktx_swa.h `ktx_resid_norm`)
     adds a sublayer's output (optionally unit-RMS-normed with a weight vector first) and a mixture's weighted expert rows to x, norms
     the updated rows and — when a causal input convolution follows (`conv=`, operators/conv.py KInputConv) — lays them out with each
-    request's convolution state in front, which `ktx_input_conv` then turns into what the sublayer reads.  `rows=` gathers rows (the
-    model's last norm).  Checkpoint tensor: the module's key (a 0-d or 1-element tensor)."""
+    request's convolution state in front, which `ktx_input_conv` then turns into what the sublayer reads; a step in which every request
+    brings one token (decode) does the convolution in the norm's own launch.  `rows=` gathers rows (the model's last norm).  Checkpoint tensor: the module's key (a 0-d or 1-element tensor)."""
 
     def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda", **kwargs):
         BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
@@ -127,10 +127,12 @@ class KScalarRMSNorm(BaseInjectedModule):
     def forward(self, x, batch=None, conv=None, conv_state=None, y=None, y_norm=None, moe=None, rows=None, out_dtype=None):
         """x fp32 [T, W] (+= y, moe, in place) -> the normed rows (through `conv` when given) in out_dtype."""
         import torch
-        from ktransformers_amd._native_swa import input_conv, resid_norm
+        from ktransformers_amd._native_swa import FUSED_CONV_MAX_TAPS, input_conv, resid_norm
         dt = out_dtype or self.compute_dtype or torch.float32
         if conv is None or conv.taps <= 1:
             return resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), rows=rows, out_dtype=dt)
+        if batch.max_q_len == 1 and conv.taps <= FUSED_CONV_MAX_TAPS:      # decode steps: one launch
+            return resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), conv=(conv.weight_f32, batch, conv_state), out_dtype=dt)
         hx = resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), halo=(conv.taps - 1, batch, conv_state))
         return input_conv(hx, conv.weight_f32, batch, conv_state, out_dtype=dt)
 
