@@ -133,7 +133,27 @@ def dense_gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=torch.float32, act: s
     return out
 
 
+def dense_gemm_skinny(a: torch.Tensor, w: torch.Tensor, act: str | None = None) -> torch.Tensor:
+    """dense_gemm with an fp32 result for products with FEW output columns (a router, a low-rank projection): on prompt-sized steps their
+    64 x 64 tiles are too few to fill the chip, so K is split over workgroups that add into a zeroed result (fp32 atomics: the order of
+    the partial sums, and with it the last bit, is not fixed); the activation then has its own launch."""
+    M, K = a.shape
+    N = w.shape[0]
+    tiles = ((M + 63) // 64) * ((N + 63) // 64)
+    ks = 1
+    if M >= SKINNY_MIN_M and tiles < 256:
+        while ks < 8 and tiles * ks * 2 <= 512 and K // (ks * 2) >= 256:
+            ks *= 2
+    if ks == 1:
+        return dense_gemm(a, w, act=act)
+    y = dense_gemm(a, w, ksplit=ks)
+    if ACT[act]:
+        check(lib.ktx_gelu_tanh(y.numel(), y.data_ptr(), SEQ_DTYPE[y.dtype], _stream_ptr(y.device)))
+    return y
+
+
 LIBRARY_GEMM_MIN_M = 64
+SKINNY_MIN_M = 256
 _LIBRARY_GEMM: list = []
 
 

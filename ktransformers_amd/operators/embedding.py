@@ -134,8 +134,8 @@ class KTokenSideInput(BaseInjectedModule):
 
     def forward(self, x: torch.Tensor, tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
         """x fp32 [T, width] (the residual after the layer's sublayers), tokens int32 [T] -> y fp32 [T, width], not yet normed."""
-        from ktransformers_amd._native_seq import dense_gemm
+        from ktransformers_amd._native_seq import dense_gemm, dense_gemm_skinny
         from ktransformers_amd._native_swa import rows_mul_lookup
-        g = dense_gemm(x, self.w["gate"], act="gelu_tanh")
+        g = dense_gemm_skinny(x, self.w["gate"], act="gelu_tanh")
         ge = rows_mul_lookup(g, table, self.layer_idx * self.dim, tokens, out_dtype=self.compute_dtype)
         return dense_gemm(ge, self.w["proj"])

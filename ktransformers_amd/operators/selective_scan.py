@@ -48,13 +48,13 @@ class KSelectiveScanMixer(BaseInjectedModule):
 
     def forward(self, h: torch.Tensor, batch, cache, cache_idx: int) -> torch.Tensor:
         """h [T, width] in the compute type -> W_o(gated scan output) fp32 [T, width]; the slots' state moves on."""
-        from ktransformers_amd._native_seq import dense_gemm
+        from ktransformers_amd._native_seq import dense_gemm, dense_gemm_skinny
         from ktransformers_amd._native_swa import ssm_conv, ssm_scan
         I, N, R = self.inner, self.state, self.dt_rank
         S, cs = cache.S[cache_idx], cache.conv[cache_idx]
         proj = dense_gemm(h, self.w["in"])                                   # [x | z], fp32
         xc = ssm_conv(self._cfg, proj, 0, self.w["conv"], self.w["conv_b"], batch, cs)
-        low = dense_gemm(xc, self.w["x"])                                    # [dt_low | B | C], fp32
+        low = dense_gemm_skinny(xc, self.w["x"])                                   # [dt_low | B | C], fp32
         dt_raw = dense_gemm(low[:, :R], self.w["dt"])
         y = ssm_scan(self._cfg, xc, low[:, R:R + N], low[:, R + N:], dt_raw, self.w["dt_b"], self.w["A_log"], self.w["D"], proj, 0, I, batch,
                      S, cs, out_dtype=self.compute_dtype)

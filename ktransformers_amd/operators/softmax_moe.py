@@ -44,10 +44,10 @@ class KSoftmaxRoutedMoE(BaseInjectedModule):
         """h [T, width] in the compute type -> the pieces of the weighted sum: (expert_rows fp32 [T * top, width] in sorted order,
         pair_pos int32 [T * top], topk_idx int32 [T, top], topk_w fp32 [T, top], number of real experts, h)."""
         from ktransformers_amd._native_hyb import WIDE_MIN_ROWS_PER_EXPERT, expert_gemm, moe_plan
-        from ktransformers_amd._native_seq import dense_gemm
+        from ktransformers_amd._native_seq import dense_gemm_skinny
         from ktransformers_amd._native_swa import softmax_route
         E, R = self.experts, self.experts + self.identity
-        logits = dense_gemm(h, self.w["router"])
+        logits = dense_gemm_skinny(h, self.w["router"])
         idx, wts = softmax_route(logits, self.top, self.sum_eps, self.w["correction"])
         wide = self.compute_dtype == torch.bfloat16 and h.shape[0] * self.top >= WIDE_MIN_ROWS_PER_EXPERT * R
         plan = moe_plan(idx, R, wide=wide)
