@@ -45,7 +45,7 @@ typedef struct ktx_resid_args {
    * t + (b + 1) * halo — the layout ktx_input_conv reads.
    * conv_w (fp32 [W][conv_taps], instead of halo; same batch tensors; EVERY request brings exactly one token; 2 <= conv_taps <= 9): the
    * input convolution in the same launch — out[t] = h + conv(h) of out_dtype with h = the normed row and the slot's state before it,
-   * and the slot's state moves on by one token. */
+   * and the slot's state moves on by one token.  conv_taps == 1 (any step, no batch tensors, no state): out[t] = h + conv_w * h. */
   const float* norm_g;
   float eps;
   const int32_t* rows;

@@ -76,7 +76,8 @@ def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | N
     norm = (g: one fp32 number on the device, eps), returns x * g / rms(x) — in out_dtype [T or len(rows), W], or, with
     halo = (taps - 1, batch, conv_state [slots, taps - 1, W]), as fp32 [T + B * halo, W] with every request's state rows in front of
     its tokens (what input_conv reads).  conv = (taps weight fp32 [W, taps], batch, conv_state), for steps in which every request brings
-    exactly ONE token: h + conv(h) in out_dtype [T, W] from the same launch, the slots' state moved on."""
+    exactly ONE token: h + conv(h) in out_dtype [T, W] from the same launch, the slots' state moved on (a one-tap convolution has no
+    state and takes any step)."""
     _f32(x, "resid_norm x")
     T, W = x.shape
     a = _ResidArgs()
@@ -124,13 +125,16 @@ def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | N
             cw, batch, state = conv
             _f32(cw, "resid_norm conv weight"), _f32(state, "resid_norm conv_state")
             taps = cw.shape[1]
-            if halo is not None or rows is not None or cw.shape[0] != W or not 2 <= taps <= FUSED_CONV_MAX_TAPS or batch.max_q_len != 1 or \
-                    batch.T != T or tuple(state.shape[1:]) != (taps - 1, W):
-                raise KtxError("resid_norm: the fused convolution takes one token per request, 2 .. 9 taps, a state [slots, taps - 1, W]")
-            a.conv_w, a.conv_taps, a.B = cw.data_ptr(), taps, int(batch.B)
-            a.q_indptr, a.pos0, a.slot, a.tok_req = (batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
-                                                     batch.tok_req.data_ptr())
-            a.conv_state = state.data_ptr()
+            if halo is not None or rows is not None or cw.shape[0] != W or not 1 <= taps <= FUSED_CONV_MAX_TAPS:
+                raise KtxError("resid_norm: the fused convolution takes 1 .. 9 taps [W, taps], no halo, no row gather")
+            a.conv_w, a.conv_taps = cw.data_ptr(), taps
+            if taps > 1:
+                if batch.max_q_len != 1 or batch.T != T or state is None or tuple(state.shape[1:]) != (taps - 1, W):
+                    raise KtxError("resid_norm: beyond one tap the fused convolution takes one token per request and a state [slots, taps - 1, W]")
+                a.B = int(batch.B)
+                a.q_indptr, a.pos0, a.slot, a.tok_req = (batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(),
+                                                         batch.tok_req.data_ptr())
+                a.conv_state = state.data_ptr()
         out = torch.empty((n_out, W), dtype=out_dtype, device=x.device)
         a.out, a.out_dtype = out.data_ptr(), SEQ_DTYPE[out_dtype]
     check(lib.ktx_resid_norm(rows.numel() if rows is not None else T, W, x.data_ptr(), C.byref(a), _stream_ptr(x.device)))

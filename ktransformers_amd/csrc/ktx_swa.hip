@@ -87,9 +87,10 @@ __global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restric
   const float r = a.norm_g[0] / sqrtf(block_sum256(s, red) / (float)W + a.eps);
   OT* out = reinterpret_cast<OT*>(a.out);
   if (a.conv_w) {                // one new token per request: the convolution and the state's move happen here
-    const int b = a.tok_req[t], taps = a.conv_taps, halo = taps - 1;
-    const bool cont = a.pos0[b] > 0;
-    float* st = a.conv_state + (size_t)a.slot[b] * halo * W;
+    const int taps = a.conv_taps, halo = taps - 1;             // (one tap: no neighbours, no state)
+    const int b = halo > 0 ? a.tok_req[t] : 0;
+    const bool cont = halo > 0 && a.pos0[b] > 0;
+    float* st = halo > 0 ? a.conv_state + (size_t)a.slot[b] * halo * W : nullptr;
     for (int e = tid; e < W; e += 256) {
       const float hn = row[e] * r;
       float prev[RN_MAX_HALO];
@@ -831,9 +832,9 @@ int ktx_resid_norm(int T, int W, float* d_x, const ktx_resid_args* a, ktx_stream
   KTX_REQUIRE(a->halo <= 0 || (a->norm_g && !a->rows && a->B > 0 && a->q_indptr && a->pos0 && a->slot && a->tok_req && a->conv_state &&
                                a->out_dtype == KTX_SEQ_F32),
               "ktx_resid_norm: halo rows need the batch's tensors, the state and an fp32 output");
-  KTX_REQUIRE(!a->conv_w || (a->halo <= 0 && a->norm_g && !a->rows && a->conv_taps >= 2 && a->conv_taps <= RN_MAX_HALO + 1 && a->q_indptr &&
-                             a->pos0 && a->slot && a->tok_req && a->conv_state),
-              "ktx_resid_norm: the fused convolution needs 2 <= taps <= 9, the batch's tensors and the state, and no halo");
+  KTX_REQUIRE(!a->conv_w || (a->halo <= 0 && a->norm_g && !a->rows && a->conv_taps >= 1 && a->conv_taps <= RN_MAX_HALO + 1 &&
+                             (a->conv_taps == 1 || (a->q_indptr && a->pos0 && a->slot && a->tok_req && a->conv_state))),
+              "ktx_resid_norm: the fused convolution needs 1 <= taps <= 9, no halo and, beyond one tap, the batch's tensors and the state");
   if (T == 0 || (!adds && !a->norm_g)) return 0;
   hipStream_t st = (hipStream_t)stream;
   const size_t lds = (size_t)W * 4;

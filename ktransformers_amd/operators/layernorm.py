@@ -129,9 +129,9 @@ class KScalarRMSNorm(BaseInjectedModule):
         import torch
         from ktransformers_amd._native_swa import FUSED_CONV_MAX_TAPS, input_conv, resid_norm
         dt = out_dtype or self.compute_dtype or torch.float32
-        if conv is None or conv.taps <= 1:
+        if conv is None or conv.taps < 1:
             return resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), rows=rows, out_dtype=dt)
-        if batch.max_q_len == 1 and conv.taps <= FUSED_CONV_MAX_TAPS:      # decode steps: one launch
+        if conv.taps == 1 or (batch.max_q_len == 1 and conv.taps <= FUSED_CONV_MAX_TAPS):      # no neighbours, or decode steps: one launch
             return resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), conv=(conv.weight_f32, batch, conv_state), out_dtype=dt)
         hx = resid_norm(x, y=y, y_norm=y_norm, moe=moe, norm=(self.g, self.eps), halo=(conv.taps - 1, batch, conv_state))
         return input_conv(hx, conv.weight_f32, batch, conv_state, out_dtype=dt)

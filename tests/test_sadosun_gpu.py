@@ -91,6 +91,11 @@ CONFIGS = {
                                     R.attention_layer(heads=1, kv_heads=1, window=1, rot=False, mlp=None),
                                     R.attention_layer(heads=2, kv_heads=1, window=None, rot=False, mlp=R.moe_mlp(experts=1, top=1, identity=4))],
                                    width=24, taps=0, side=0, scale=1.0),
+    # sizes that are 1: one tap in the input convolutions, one head, a window of one, one expert, one state entry, a side input of one
+    "ones": lambda: R.make_config([R.attention_layer(heads=1, kv_heads=1, dim=2, vdim=2, window=1, rot_dims=2, mlp=R.moe_mlp(experts=1, top=1, identity=0, ff=1)),
+                                   R.scan_layer(inner=1, state=1, dt_rank=1, conv=1, mlp=R.moe_mlp(experts=1, top=2, identity=1, ff=3)),
+                                   R.attention_layer(heads=2, kv_heads=1, dim=4, vdim=2, window=2, rot_dims=0, mlp=None)],
+                                  width=8, vocab=9, taps=1, side=1, scale=1.0),
 }
 
 
@@ -120,16 +125,16 @@ def batch_of(lens, pos0=None, slots=None, page_size=16, pages=None):
 
 
 # ---- mechanisms alone ----------------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("W,taps", [(48, 3), (37, 2), (300, 4), (5000, 3), (64, 1)])
+@pytest.mark.parametrize("W,taps", [(48, 3), (37, 2), (300, 4), (5000, 3), (64, 0), (40, 1), (24, 9), (16, 10)])
 def test_scalar_norm_residual_update_and_input_convolution(W, taps):
     from ktransformers_amd._native_swa import input_conv, resid_norm
     g = torch.Generator().manual_seed(W)
     eps, gw = 1e-3, torch.tensor([1.3])
-    w = torch.randn(W, taps, generator=g) * 0.5
+    w = torch.randn(W, max(taps, 1), generator=g) * 0.5
     lens = [7, 1, 12]
     seqs = [torch.randn(n, W, generator=g) * 3 + 0.5 for n in lens]
     ys = [torch.randn(n, W, generator=g) for n in lens]
-    want = [R.input_conv(R.scalar_norm((s + y).double(), gw.double(), eps), w.double()) if taps > 1 else R.scalar_norm((s + y).double(), gw.double(), eps)
+    want = [R.input_conv(R.scalar_norm((s + y).double(), gw.double(), eps), w.double()) if taps else R.scalar_norm((s + y).double(), gw.double(), eps)
             for s, y in zip(seqs, ys)]
     # whole sequences in one batch, then the same cut in two steps with the state carried in slots that held garbage
     for cuts in ([0], [0, 3], [0, 1, 2], [0, 1, 2, 3, 4, 5]):
@@ -144,8 +149,8 @@ def test_scalar_norm_residual_update_and_input_convolution(W, taps):
             fb = batch_of([bounds[b][k + 1] - bounds[b][k] for b in live], pos0=[bounds[b][k] for b in live], slots=[slots[b] for b in live])
             x = torch.cat([seqs[b][bounds[b][k]:bounds[b][k + 1]] for b in live]).to(DEV)
             y = torch.cat([ys[b][bounds[b][k]:bounds[b][k + 1]] for b in live]).to(DEV)
-            if taps > 1 and fb.max_q_len == 1:        # one token per request: the convolution rides in the norm's launch
-                h = resid_norm(x, y=y, norm=(gw.to(DEV), eps), conv=(w.to(DEV), fb, state))
+            if taps == 1 or (1 < taps <= 9 and fb.max_q_len == 1):    # no neighbours, or one token per request: the norm's own launch
+                h = resid_norm(x, y=y, norm=(gw.to(DEV), eps), conv=(w.to(DEV), fb, state if taps > 1 else None))
             elif taps > 1:
                 hx = resid_norm(x, y=y, norm=(gw.to(DEV), eps), halo=(taps - 1, fb, state))
                 h = input_conv(hx, w.to(DEV), fb, state)
@@ -212,8 +217,8 @@ def attn_weights(c, W, g, boost=1.0):
             "mix.o": m(W, H * V, 1 / math.sqrt(H * V))}
 
 
-ATTN_SIZES = [  # heads, kv_heads, dim, vdim, window, rot_dims (None: all of dim; -1: no rotation at all)
-    (4, 2, 16, 16, 12, None), (3, 1, 10, 6, 5, 4), (6, 3, 12, 80, None, None), (1, 1, 16, 16, 1, None), (2, 1, 24, 8, 9, -1),
+ATTN_SIZES = [  # heads, kv_heads, dim, vdim, window, rot_dims (None: all of dim; 0: values turn, q and k do not; -1: no rotation at all)
+    (4, 2, 16, 16, 12, None), (2, 1, 16, 8, 9, 0), (2, 2, 32, 32, 9, 0), (3, 1, 10, 6, 5, 4), (6, 3, 12, 80, None, None), (1, 1, 16, 16, 1, None), (2, 1, 24, 8, 9, -1),
     (8, 2, 32, 64, 24, None), (4, 4, 64, 32, None, 32), (16, 1, 32, 32, 40, 16), (2, 2, 96, 96, 20, None), (4, 1, 128, 128, 33, 64),
     (2, 1, 256, 256, 17, None)]
 
@@ -387,7 +392,7 @@ def test_softmax_router(E, top, T):
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
 @pytest.mark.parametrize("E,ID,top,F,T", [(5, 2, 2, 24, 50), (3, 0, 1, 7, 9), (4, 2, 6, 32, 130), (16, 1, 3, 40, 1), (2, 1, 2, 136, 400),
-                                          (1, 4, 1, 16, 20), (8, 0, 2, 64, 3)])
+                                          (1, 4, 1, 16, 20), (8, 0, 2, 64, 3), (12, 3, 11, 16, 30), (20, 0, 17, 8, 2)])
 def test_mixture_with_identity_experts(dtype, E, ID, top, F, T):
     """The operator's pieces, joined by the residual update, against the plain mixture: streaming products (few pairs), 64-row tiles
     and 128-row tiles (many pairs per expert), tokens whose choices are all identity experts."""
@@ -459,7 +464,7 @@ def test_whole_prompt_and_layers(dtype, name):
 
 
 @pytest.mark.parametrize("dtype", [F32, BF16])
-@pytest.mark.parametrize("name", ["mixed", "odd", "wide"])
+@pytest.mark.parametrize("name", ["mixed", "odd", "wide", "ones"])
 def test_prefill_equals_token_by_token_and_portions(dtype, name):
     cfg = CONFIGS[name]()
     model, cache, P = build(cfg, 12, dtype, page_size=8)
