@@ -2044,7 +2044,7 @@ class SwaRandomLoader(HybRandomLoader):
 class SwaKernelTimer(HybKernelTimer):
     """HIP events around every call of the window-attention / scan bindings and of the shared grouped and dense products."""
     HYB = ("moe_plan", "expert_gemm")
-    SWA = ("resid_norm", "input_conv", "rows_mul_lookup", "swa_prep", "swa_forward", "swa_mfma", "ssm_conv", "ssm_scan", "softmax_route")
+    SWA = ("resid_norm", "input_conv", "rows_mul_lookup", "swa_prep", "swa_forward", "swa_mfma", "ssm_conv", "ssm_scan", "softmax_route", "softmax_route_plan")
 
     def _cost(self, name, a, kw, out):
         nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0

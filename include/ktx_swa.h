@@ -142,6 +142,14 @@ int ktx_ssm_scan(const ktx_ssm_config* cfg, int B, int T, int max_q_len, const i
 int ktx_softmax_route(int T, int E, int top, float sum_eps, const float* d_logits, int64_t ldl, const float* d_correction,
                       int32_t* d_topk_idx, float* d_topk_w, ktx_stream_t stream);
 
+/* The same router followed, in the same launch, by the expert sort of ktx_moe_plan (ktx_hyb.h; same outputs, E groups): for small steps
+ * (decode), T <= KTX_ROUTE_PLAN_MAX_T, where one workgroup routes and sorts. */
+enum { KTX_ROUTE_PLAN_MAX_T = 256 };
+int ktx_softmax_route_plan(int T, int E, int top, float sum_eps, const float* d_logits, int64_t ldl, const float* d_correction,
+                           int32_t* d_topk_idx, float* d_topk_w, int tile_m, int32_t* d_group_off, int32_t* d_sorted_tok,
+                           int32_t* d_pair_pos, int32_t* d_sorted_group, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles,
+                           ktx_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -42,6 +42,7 @@ lib.ktx_ssm_conv.argtypes = [C.POINTER(_SsmConfig), _I, _I, _P, _P, _P, _P, _P, 
 lib.ktx_ssm_scan.argtypes = [C.POINTER(_SsmConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _P, _P, _P,
                              _I, _P]
 lib.ktx_softmax_route.argtypes = [_I, _I, _I, _F, _P, _L, _P, _P, _P, _P]
+lib.ktx_softmax_route_plan.argtypes = [_I, _I, _I, _F, _P, _L, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P]
 
 
 FUSED_CONV_MAX_TAPS = 9      # ktx_resid_norm's one-token form keeps the state rows of one channel in registers
@@ -280,3 +281,32 @@ def softmax_route(logits: torch.Tensor, top: int, sum_eps: float, correction: to
     w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
     check(lib.ktx_softmax_route(T, E, top, float(sum_eps), lp, ldl, _ptr(correction), idx.data_ptr(), w.data_ptr(), _stream_ptr(logits.device)))
     return idx, w
+
+
+ROUTE_PLAN_MAX_T = 64        # up to this many tokens a step routes and sorts in one launch (ktx_softmax_route_plan takes up to 256)
+
+
+def softmax_route_plan(logits: torch.Tensor, top: int, sum_eps: float, correction: torch.Tensor | None = None):
+    """softmax_route and the expert sort over all E router outputs (ktransformers_amd._native_hyb.moe_plan, 64-row tiles) in ONE launch,
+    for small steps -> (topk_idx, topk_w, plan)."""
+    from ktransformers_amd._native_hyb import TILE_M, MoePlan
+    lp, ldl = _rows_f32(logits, "softmax_route_plan logits")
+    _f32(correction, "softmax_route_plan correction")
+    T, E = logits.shape
+    if correction is not None and correction.numel() != E:
+        raise KtxError("softmax_route_plan: one correction per router output")
+    idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
+    w = torch.empty((T, top), dtype=torch.float32, device=logits.device)
+    p = MoePlan()
+    p.pairs, p.tile_m = T * top, TILE_M
+    p.max_tiles = p.pairs // p.tile_m + min(E, p.pairs) + 1
+    meta = torch.empty(E + 1 + 3 * p.pairs + 2 * p.max_tiles + 1, dtype=torch.int32, device=logits.device)
+    at = 0
+    for name, n in (("group_off", E + 1), ("sorted_tok", p.pairs), ("pair_pos", p.pairs), ("sorted_group", p.pairs), ("tile_group", p.max_tiles),
+                    ("tile_row0", p.max_tiles), ("num_tiles", 1)):
+        setattr(p, name, meta[at:at + n])
+        at += n
+    check(lib.ktx_softmax_route_plan(T, E, top, float(sum_eps), lp, ldl, _ptr(correction), idx.data_ptr(), w.data_ptr(), p.tile_m,
+                                     p.group_off.data_ptr(), p.sorted_tok.data_ptr(), p.pair_pos.data_ptr(), p.sorted_group.data_ptr(),
+                                     p.tile_group.data_ptr(), p.tile_row0.data_ptr(), p.num_tiles.data_ptr(), _stream_ptr(logits.device)))
+    return idx, w, p

@@ -769,44 +769,14 @@ __global__ void __launch_bounds__(256) moe_route_kernel(int T, int E, int top, f
   for (int k = lane; k < top; k += 64) wts[(size_t)t * top + k] *= f;
 }
 
-// one workgroup sorts the pairs by expert (counting sort in LDS) and lays the row tiles out
+// one workgroup sorts the pairs by expert (counting sort in LDS) and lays the row tiles out (moe_plan_block, ktx_seq_dev.inc)
 __global__ void __launch_bounds__(1024) moe_plan_kernel(int pairs, int E, int top, int tile_m, const int32_t* __restrict__ idx,
                                                         int32_t* __restrict__ group_off, int32_t* __restrict__ sorted_tok,
                                                         int32_t* __restrict__ pair_pos, int32_t* __restrict__ sorted_group,
                                                         int32_t* __restrict__ tile_group, int32_t* __restrict__ tile_row0,
                                                         int32_t* __restrict__ num_tiles) {
   extern __shared__ int32_t pl[];          // counts [E] | offsets [E + 1] | cursor [E]
-  int32_t* cnt = pl;
-  int32_t* off = pl + E;
-  int32_t* cur = off + E + 1;
-  const int tid = threadIdx.x;
-  for (int e = tid; e < E; e += 1024) cnt[e] = cur[e] = 0;
-  __syncthreads();
-  for (int i = tid; i < pairs; i += 1024) atomicAdd(&cnt[idx[i]], 1);
-  __syncthreads();
-  if (tid == 0) {
-    int at = 0, nt = 0;
-    for (int e = 0; e < E; e++) {
-      off[e] = at;
-      for (int r = 0; r < cnt[e]; r += tile_m) {
-        tile_group[nt] = e;
-        tile_row0[nt] = at + r;
-        nt++;
-      }
-      at += cnt[e];
-    }
-    off[E] = at;
-    num_tiles[0] = nt;
-  }
-  __syncthreads();
-  for (int e = tid; e <= E; e += 1024) group_off[e] = off[e];
-  for (int i = tid; i < pairs; i += 1024) {
-    const int e = idx[i];
-    const int p = off[e] + atomicAdd(&cur[e], 1);
-    sorted_tok[p] = i / top;
-    sorted_group[p] = e;
-    pair_pos[i] = p;
-  }
+  moe_plan_block(pairs, E, top, tile_m, idx, group_off, sorted_tok, pair_pos, sorted_group, tile_group, tile_row0, num_tiles, pl);
 }
 
 // ---------------------------------------------------------------------------------------------------------------------

@@ -749,11 +749,8 @@ __global__ void __launch_bounds__(256) ssm_scan_kernel(ktx_ssm_config c, const i
 // ---------------------------------------------------------------------------------------------------------------------
 // router: one wavefront per token; lane holds outputs lane, lane + 64, ... (E <= 64 * SR_RE)
 constexpr int SR_RE = 16;
-__global__ void __launch_bounds__(256) softmax_route_kernel(int T, int E, int top, float sum_eps, const float* __restrict__ logits,
-                                                            int64_t ldl, const float* __restrict__ corr, int32_t* __restrict__ idx,
-                                                            float* __restrict__ wts) {
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
-  if (t >= T) return;
+__device__ __forceinline__ void softmax_route_token(int t, int lane, int E, int top, float sum_eps, const float* __restrict__ logits,
+                                                    int64_t ldl, const float* __restrict__ corr, int32_t* idx, float* wts) {
   float s[SR_RE], ch[SR_RE];
   float mx = -INFINITY;
 #pragma unroll
@@ -814,6 +811,28 @@ __global__ void __launch_bounds__(256) softmax_route_kernel(int T, int E, int to
   __builtin_amdgcn_wave_barrier();
   if (lane == 0)
     for (int k = 0; k < top; k++) wts[(size_t)t * top + k] *= f;
+}
+
+__global__ void __launch_bounds__(256) softmax_route_kernel(int T, int E, int top, float sum_eps, const float* __restrict__ logits,
+                                                            int64_t ldl, const float* __restrict__ corr, int32_t* __restrict__ idx,
+                                                            float* __restrict__ wts) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+  if (t < T) softmax_route_token(t, lane, E, top, sum_eps, logits, ldl, corr, idx, wts);
+}
+
+// router and expert sort of a SMALL step (decode) in one launch: the sixteen wavefronts of the one workgroup route the tokens, then the
+// workgroup sorts the pairs it has just written (moe_plan_block)
+__global__ void __launch_bounds__(1024) softmax_route_plan_kernel(int T, int E, int top, float sum_eps, const float* __restrict__ logits,
+                                                                  int64_t ldl, const float* __restrict__ corr, int32_t* idx, float* wts,
+                                                                  int tile_m, int32_t* __restrict__ group_off,
+                                                                  int32_t* __restrict__ sorted_tok, int32_t* __restrict__ pair_pos,
+                                                                  int32_t* __restrict__ sorted_group, int32_t* __restrict__ tile_group,
+                                                                  int32_t* __restrict__ tile_row0, int32_t* __restrict__ num_tiles) {
+  extern __shared__ int32_t pl[];          // counts [E] | offsets [E + 1] | cursor [E]
+  for (int t = threadIdx.x >> 6; t < T; t += 16) softmax_route_token(t, threadIdx.x & 63, E, top, sum_eps, logits, ldl, corr, idx, wts);
+  __threadfence_block();
+  __syncthreads();
+  moe_plan_block(T * top, E, top, tile_m, idx, group_off, sorted_tok, pair_pos, sorted_group, tile_group, tile_row0, num_tiles, pl);
 }
 
 }  // namespace
@@ -1094,6 +1113,21 @@ int ktx_softmax_route(int T, int E, int top, float sum_eps, const float* d_logit
               "ktx_softmax_route: 0 < top <= outputs <= 1024");
   if (T == 0) return 0;
   softmax_route_kernel<<<(T + 3) / 4, 256, 0, (hipStream_t)stream>>>(T, E, top, sum_eps, d_logits, ldl, d_correction, d_topk_idx, d_topk_w);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_softmax_route_plan(int T, int E, int top, float sum_eps, const float* d_logits, int64_t ldl, const float* d_correction,
+                           int32_t* d_topk_idx, float* d_topk_w, int tile_m, int32_t* d_group_off, int32_t* d_sorted_tok,
+                           int32_t* d_pair_pos, int32_t* d_sorted_group, int32_t* d_tile_group, int32_t* d_tile_row0, int32_t* d_num_tiles,
+                           ktx_stream_t stream) {
+  KTX_REQUIRE(T >= 0 && T <= KTX_ROUTE_PLAN_MAX_T && E > 0 && top > 0 && top <= E && E <= 64 * SR_RE && d_logits && d_topk_idx && d_topk_w &&
+                  ldl >= E && tile_m > 0 && d_group_off && d_sorted_tok && d_pair_pos && d_sorted_group && d_tile_group && d_tile_row0 &&
+                  d_num_tiles,
+              "ktx_softmax_route_plan: a small step (T <= 256), 0 < top <= outputs <= 1024, pointers");
+  softmax_route_plan_kernel<<<1, 1024, (size_t)(3 * E + 1) * 4, (hipStream_t)stream>>>(
+      T, E, top, sum_eps, d_logits, ldl, d_correction, d_topk_idx, d_topk_w, tile_m, d_group_off, d_sorted_tok, d_pair_pos, d_sorted_group,
+      d_tile_group, d_tile_row0, d_num_tiles);
   KTX_HIP(hipGetLastError());
   return 0;
 }

@@ -5,7 +5,8 @@ operator beside operators/sigmoid_moe.py (sigmoid scores, GLU experts) and the q
     weights are s (without the correction) over (the chosen s' sum + 1e-20);  expert e: W_down relu(W_up h)^2, no biases;  the LAST
     `identity` router outputs stand for experts without weights that return h itself.
 
-The real experts run as two grouped products over the (token, choice) pairs sorted by router output (include/ktx_hyb.h `ktx_moe_plan`,
+The real experts run as two grouped products over the (token, choice) pairs sorted by router output (include/ktx_hyb.h `ktx_moe_plan`; small
+steps route and sort in one launch, `ktx_softmax_route_plan`;
 `ktx_grouped_gemm` / `ktx_grouped_gemv` with the relu^2 epilogue; groups beyond the real experts are skipped); the weighted sum over a
 token's choices — rows of real experts, h for identity ones — is left to the consumer's launch (`ktx_resid_norm`), so forward returns the
 pieces.  top, identity and the sum's eps are constructor arguments (read from the replaced module).  Checkpoint tensors:
@@ -45,12 +46,15 @@ class KSoftmaxRoutedMoE(BaseInjectedModule):
         pair_pos int32 [T * top], topk_idx int32 [T, top], topk_w fp32 [T, top], number of real experts, h)."""
         from ktransformers_amd._native_hyb import WIDE_MIN_ROWS_PER_EXPERT, expert_gemm, moe_plan
         from ktransformers_amd._native_seq import dense_gemm_skinny
-        from ktransformers_amd._native_swa import softmax_route
+        from ktransformers_amd._native_swa import ROUTE_PLAN_MAX_T, softmax_route, softmax_route_plan
         E, R = self.experts, self.experts + self.identity
         logits = dense_gemm_skinny(h, self.w["router"])
-        idx, wts = softmax_route(logits, self.top, self.sum_eps, self.w["correction"])
-        wide = self.compute_dtype == torch.bfloat16 and h.shape[0] * self.top >= WIDE_MIN_ROWS_PER_EXPERT * R
-        plan = moe_plan(idx, R, wide=wide)
+        if h.shape[0] <= ROUTE_PLAN_MAX_T:       # decode steps: router and sort in one launch
+            idx, wts, plan = softmax_route_plan(logits, self.top, self.sum_eps, self.w["correction"])
+        else:
+            idx, wts = softmax_route(logits, self.top, self.sum_eps, self.w["correction"])
+            wide = self.compute_dtype == torch.bfloat16 and h.shape[0] * self.top >= WIDE_MIN_ROWS_PER_EXPERT * R
+            plan = moe_plan(idx, R, wide=wide)
         act = expert_gemm(h, self.w["up"], plan, gather=True, out_dtype=self.compute_dtype, act="relu_sq")
         rows = expert_gemm(act, self.w["down"], plan, gather=False)
         return rows, plan.pair_pos, idx, wts, E, h

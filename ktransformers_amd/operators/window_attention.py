@@ -7,7 +7,7 @@ operators (operators/attention.py, latent_window_attention.py) for decoders on a
     the value of position j is turned by j over ALL its entries (pairs (2m, 2m + 1), angle j base^(-2m / vdim)) and cached so; a
     head's weighted sum at position i is turned back by i — values enter relative to the query;
     score = scale (q . k); position i sees j with 0 <= i - j < window;
-    weights p_j = exp(s_j) / (e^sink + sum_j exp(s_j)): a sink without a value in the denominator (score 0: "one added");
+    weights p_j = exp(s_j) / (e^sink + sum_j exp(s_j)): a sink that takes weight and gives no value (with score 0 the extra term is 1);
     W_o on the concatenated heads.
 
 Rotated, normed keys and rotated values are appended to the KHybridCache's paged key / value caches (spec "kv") by the prep launch;

@@ -378,6 +378,20 @@ def test_softmax_router(E, top, T):
         assert torch.equal(idx.cpu().long().sort(dim=1).values, ridx.sort(dim=1).values)
         order = idx.cpu().long().argsort(dim=1), ridx.argsort(dim=1)
         assert rel(torch.gather(w.cpu(), 1, order[0]), torch.gather(rw, 1, order[1])) < 1e-6
+    if T <= 64:      # small steps route and sort in one launch: the same choices, and a sort that puts every pair into its expert's rows
+        from ktransformers_amd._native_hyb import moe_plan
+        from ktransformers_amd._native_swa import softmax_route_plan
+        zc = z.to(DEV)[:, :E].contiguous()
+        idx1, w1 = softmax_route(zc, top, 1e-20, corr.to(DEV))
+        idx2, w2, plan = softmax_route_plan(zc, top, 1e-20, corr.to(DEV))
+        assert torch.equal(idx1, idx2) and torch.equal(w1, w2)
+        ref_plan = moe_plan(idx1, E)
+        assert torch.equal(plan.group_off, ref_plan.group_off) and int(plan.num_tiles) == int(ref_plan.num_tiles)
+        nt = int(plan.num_tiles)
+        assert torch.equal(plan.tile_group[:nt], ref_plan.tile_group[:nt]) and torch.equal(plan.tile_row0[:nt], ref_plan.tile_row0[:nt])
+        flat, pos = idx2.reshape(-1).long(), plan.pair_pos.long()
+        assert sorted(pos.tolist()) == list(range(T * top))
+        assert torch.equal(plan.sorted_group.long()[pos], flat) and torch.equal(plan.sorted_tok.long()[pos], torch.arange(T * top, device=DEV) // top)
     # the correction changes the choice, not the weights: a large one on output 0 forces it in, its weight stays its softmax share
     big = torch.zeros(E)
     big[0] = 10.0
