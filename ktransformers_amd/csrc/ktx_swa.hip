@@ -91,22 +91,39 @@ __global__ void __launch_bounds__(256) resid_norm_kernel(int W, float* __restric
     const int b = halo > 0 ? a.tok_req[t] : 0;
     const bool cont = halo > 0 && a.pos0[b] > 0;
     float* st = halo > 0 ? a.conv_state + (size_t)a.slot[b] * halo * W : nullptr;
-    for (int e = tid; e < W; e += 256) {
-      const float hn = row[e] * r;
-      float prev[RN_MAX_HALO];
-      float acc = 0.f;
+    // four channels per thread at a time, every load of the batch in front of its first store: the state is read and written through
+    // the same pointer, and a store in front of the next channel's loads would make each channel wait for a memory round trip
+    constexpr int RN_CB = 4;
+    const float* __restrict__ cw = a.conv_w;
+    for (int e0 = tid; e0 < W; e0 += 256 * RN_CB) {
+      float prev[RN_CB][RN_MAX_HALO], wv[RN_CB][RN_MAX_HALO + 1];
 #pragma unroll
-      for (int j = 0; j < RN_MAX_HALO; j++) {
-        if (j < halo) {
-          prev[j] = cont ? st[(size_t)j * W + e] : 0.f;
-          acc += a.conv_w[(size_t)e * taps + j] * prev[j];
+      for (int u = 0; u < RN_CB; u++) {
+        const int e = e0 + u * 256;
+#pragma unroll
+        for (int j = 0; j < RN_MAX_HALO; j++) {
+          const bool ok = e < W && j < halo;
+          prev[u][j] = ok && cont ? st[(size_t)j * W + e] : 0.f;
+          wv[u][j] = ok ? cw[(size_t)e * taps + j] : 0.f;
+        }
+        wv[u][RN_MAX_HALO] = e < W ? cw[(size_t)e * taps + halo] : 0.f;
+      }
+#pragma unroll
+      for (int u = 0; u < RN_CB; u++) {
+        const int e = e0 + u * 256;
+        if (e < W) {
+          const float hn = row[e] * r;
+          float acc = 0.f;
+#pragma unroll
+          for (int j = 0; j < RN_MAX_HALO; j++)
+            if (j < halo) acc += wv[u][j] * prev[u][j];
+          acc += wv[u][RN_MAX_HALO] * hn;
+          st_elem(out, (size_t)t * W + e, hn + acc);
+#pragma unroll
+          for (int j = 0; j < RN_MAX_HALO; j++)
+            if (j < halo) st[(size_t)j * W + e] = j + 1 < halo ? prev[u][(j + 1) % RN_MAX_HALO] : hn;
         }
       }
-      acc += a.conv_w[(size_t)e * taps + halo] * hn;
-      st_elem(out, (size_t)t * W + e, hn + acc);
-#pragma unroll
-      for (int j = 0; j < RN_MAX_HALO; j++)
-        if (j < halo) st[(size_t)j * W + e] = j + 1 < halo ? prev[(j + 1) % RN_MAX_HALO] : hn;
     }
     return;
   }
@@ -161,19 +178,27 @@ __global__ void __launch_bounds__(256) swa_prep_kernel(ktx_swa_config c, const f
                                                        const int32_t* __restrict__ pos, const int32_t* __restrict__ cache_loc,
                                                        KT* __restrict__ kcache, KT* __restrict__ vcache, float* __restrict__ q_out,
                                                        float* __restrict__ vcs) {
-  extern __shared__ float cs[];            // cos | sin of the rot_dims / 2 key angles, then cos | sin of the vdim / 2 value angles
+  extern __shared__ float cs[];            // cos | sin of the rot_dims / 2 key angles, cos | sin of the vdim / 2 value angles, the token's q | k | v
   const int t = blockIdx.x, tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int NP = c.rot_dims / 2, NV = c.rot_values ? c.vdim / 2 : 0;
+  const int D = c.dim, V = c.vdim, H = c.heads, G = c.kv_heads;
   float* vc = cs + 2 * NP;
+  float* row = vc + 2 * NV;                // [H * D | G * D | G * V]: read once, coalesced; the heads' passes below stay in LDS
+  const float* base = proj + (size_t)t * ldp;
+  const int nq = H * D, nk = G * D, nv = G * V;
+  for (int i = tid; i < nq + nk + nv; i += 256)
+    row[i] = base[i < nq ? q_off + i : i < nq + nk ? k_off + (i - nq) : v_off + (i - nq - nk)];
   const double p = (double)pos[t];
   for (int i = tid; i < NP; i += 256) {
-    const double a = p * inv_freq[i];
-    cs[i] = (float)cos(a);
-    cs[NP + i] = (float)sin(a);
+    double si, co;
+    sincos(p * inv_freq[i], &si, &co);
+    cs[i] = (float)co;
+    cs[NP + i] = (float)si;
   }
   for (int i = tid; i < NV; i += 256) {
-    const double a = p * v_inv_freq[i];
-    const float co = (float)cos(a), si = (float)sin(a);
+    double sd, cd;
+    sincos(p * v_inv_freq[i], &sd, &cd);
+    const float co = (float)cd, si = (float)sd;
     vc[i] = co;
     vc[NV + i] = si;
     vcs[(size_t)t * c.vdim + i] = co;
@@ -187,13 +212,11 @@ __global__ void __launch_bounds__(256) swa_prep_kernel(ktx_swa_config c, const f
     const float a = v[2 * i], bb = v[2 * i + 1];
     return (j & 1) ? bb * tab[i] + a * tab[np + i] : a * tab[i] - bb * tab[np + i];
   };
-  const float* base = proj + (size_t)t * ldp;
-  const int D = c.dim, V = c.vdim, H = c.heads, G = c.kv_heads;
   const size_t loc = (size_t)cache_loc[t];
   for (int u = wave; u < H + 2 * G; u += 4) {
     if (u < H + G) {        // a query or key head: rotate, then norm
       const bool isq = u < H;
-      const float* v = base + (isq ? q_off + (size_t)u * D : k_off + (size_t)(u - H) * D);
+      const float* v = row + (size_t)u * D;      // (key heads follow the query heads in the row)
       float r = 1.0f;
       if (c.qk_norm) {
         float s = 0.f;
@@ -213,7 +236,7 @@ __global__ void __launch_bounds__(256) swa_prep_kernel(ktx_swa_config c, const f
       }
     } else {
       const int g = u - H - G;
-      const float* v = base + v_off + (size_t)g * V;
+      const float* v = row + nq + nk + (size_t)g * V;
       KT* o = vcache + (loc * G + g) * V;
       for (int j = lane; j < V; j += 64) st_elem(o, j, turned(v, j, NV, vc));
     }
@@ -928,8 +951,11 @@ int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t 
   KTX_REQUIRE(cfg->rot_dims == 0 || d_inv_freq, "ktx_swa_prep: rotation without frequencies");
   KTX_REQUIRE(!cfg->rot_values || (d_v_inv_freq && d_vcs), "ktx_swa_prep: rotated values need their frequencies and the table");
   if (T == 0) return 0;
-  const size_t lds = ((size_t)cfg->rot_dims + (cfg->rot_values ? cfg->vdim : 0) + 2) * 4;
-  KTX_REQUIRE(lds <= 60 * 1024, "ktx_swa_prep: the angle tables must fit the LDS");
+  const size_t lds = ((size_t)cfg->rot_dims + (cfg->rot_values ? cfg->vdim : 0) + (size_t)cfg->heads * cfg->dim +
+                      (size_t)cfg->kv_heads * (cfg->dim + cfg->vdim) + 2) * 4;
+  KTX_REQUIRE(lds <= 150 * 1024, "ktx_swa_prep: a token's q | k | v row and the angle tables must fit the LDS");
+  KTX_HIP(ktx_set_max_lds((const void*)swa_prep_kernel<float>, 150 * 1024));
+  KTX_HIP(ktx_set_max_lds((const void*)swa_prep_kernel<bf16_t>, 150 * 1024));
   hipStream_t st = (hipStream_t)stream;
   if (cfg->cache_dtype == KTX_SEQ_F32)
     swa_prep_kernel<float><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, q_off, k_off, v_off, d_inv_freq, d_v_inv_freq, d_pos, d_cache_loc,
