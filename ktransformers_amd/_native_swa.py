@@ -82,7 +82,6 @@ def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | N
     _f32(x, "resid_norm x")
     T, W = x.shape
     a = _ResidArgs()
-    keep = []
     if y is not None:
         a.y, a.ldy = _rows_f32(y, "resid_norm y")
         if tuple(y.shape) != (T, W):
@@ -139,7 +138,6 @@ def resid_norm(x: torch.Tensor, y: torch.Tensor | None = None, y_norm: tuple | N
         out = torch.empty((n_out, W), dtype=out_dtype, device=x.device)
         a.out, a.out_dtype = out.data_ptr(), SEQ_DTYPE[out_dtype]
     check(lib.ktx_resid_norm(rows.numel() if rows is not None else T, W, x.data_ptr(), C.byref(a), _stream_ptr(x.device)))
-    del keep
     return out
 
 
