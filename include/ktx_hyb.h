@@ -38,6 +38,29 @@ int ktx_gated_norm_add(int T, int W, const float* d_y, int64_t ldy, const float*
                        const float* d_bn, float eps, float* d_x, const float* d_next_w, const float* d_next_b, float next_eps,
                        void* d_next_out, int next_dtype, ktx_stream_t stream);
 
+/* The post-normed residual update of one sublayer with a scaled residual, and the depth-weighted average behind a layer, one launch:
+ *   v[t] = layer_norm(alpha * x_in[t] + (y ? y[t] : 0) + (ybias ? ybias : 0); w, b, eps)
+ *   stack (fp32, level l at stack + l * stack_stride, [T][W] each; optional): level `level` receives v[t]
+ *   dwa (fp32 [level + 1], needs stack): x_out[t] = sum_{j <= level} dwa[j] * stack level j [t]; otherwise x_out[t] = v[t]
+ *   out_lp (optional, [T][W] of out_dtype): a copy of x_out for the products that follow.
+ * x_in and x_out may be the same rows (in place) or not (x_in may be a level of the stack). */
+typedef struct ktx_postnorm_args {
+  const float* y;
+  int64_t ldy;
+  const float* ybias;
+  float alpha;
+  const float* w;
+  const float* b;
+  float eps;
+  float* stack;
+  int64_t stack_stride;
+  int32_t level;
+  const float* dwa;
+  void* out_lp;
+  int32_t out_dtype;
+} ktx_postnorm_args;
+int ktx_postnorm_mix(int T, int W, const float* d_x_in, float* d_x_out, const ktx_postnorm_args* a, ktx_stream_t stream);
+
 /* PolyNorm: with u(v) = v / sqrt(mean(v^2) + eps) over a row of F values and z = in[t] + bias,
  * out[t] = c[0] u(z) + c[1] u(z^2) + c[2] u(z^3) + c[3] (powers element-wise).  in fp32 rows of stride ldz; coef fp32 [4] on the device. */
 int ktx_poly_norm(int T, int F, const float* d_z, int64_t ldz, const float* d_bias, const float* d_coef, float eps, void* d_out,
@@ -45,6 +68,17 @@ int ktx_poly_norm(int T, int F, const float* d_z, int64_t ldz, const float* d_bi
 
 /* out[r][f] = silu(in[r][f]) * in[r][F + f]: fp32 rows of 2F (stride ldi) -> [R][F] of out_dtype. */
 int ktx_silu_mul_rows(int R, int F, const float* d_in, int64_t ldi, void* d_out, int out_dtype, ktx_stream_t stream);
+
+/* out[r][f] = g * sigmoid(slope * g) * (u + up_shift) with g = min(in[r][f], limit), u = clamp(in[r][F + f], -limit, limit): the
+ * activation of a GLU whose gate is capped from above and whose linear half is clamped (limit = INFINITY: neither); fp32 rows of 2F
+ * (stride ldi) -> [R][F] of out_dtype. */
+int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, void* d_out, int out_dtype,
+                       ktx_stream_t stream);
+
+/* out[r][c] = o[r][c] * sigmoid(gate[r][c]): o [R][N] of o_dtype, gate fp32 rows of stride ldg -> [R][N] of out_dtype (an output gate
+ * on an attention's concatenated heads). */
+int ktx_sigmoid_gate_rows(int R, int N, const void* d_o, int o_dtype, const float* d_gate, int64_t ldg, void* d_out, int out_dtype,
+                          ktx_stream_t stream);
 
 /* out[t][h][v] = o[t][h][v] / sqrt(mean_v(o[t][h]^2) + eps) * w[(w_per_head ? h * vdim : 0) + v] * act(gate[t][h * vdim + v]);
  * act = sigmoid (0) or silu (1).  o fp32 [T][heads * vdim]; gate fp32 rows of stride ldg. */
@@ -84,19 +118,21 @@ typedef struct ktx_latattn_config {
   int32_t window;                             /* position i sees j with 0 <= i - j < window; <= 0: no window */
   float eps;                                  /* of the latent's RMS norm */
   int32_t page_size, cache_dtype;             /* cache rows [rows][kv_rank + rot_dim] of KTX_SEQ_* */
+  int32_t rot_half;                           /* != 0: the turning pairs are (i, i + rot_dims / 2) instead of (2i, 2i + 1) */
 } ktx_latattn_config;
 
 /* Per token: the first kv_rank entries of the down projection, RMS-normed with weight wn, and the last rot_dim, rotated at the token's
  * position (angle = pos * inv_freq[i], fp64 [rot_dims / 2]), go to cache row cache_loc[t]; each head's rotated query part goes, rotated,
  * to q_out[t][h][kv_rank ..] (q_out fp32 [T][heads][kv_rank + rot_dim]; the first kv_rank entries per head are written by the caller:
  * the un-rotated query part times W_uk of the head).  proj fp32 rows of stride ldp: q at q_off [heads][dim + rot_dim], the down
- * projection at c_off [kv_rank + rot_dim]. */
+ * projection at c_off [kv_rank + rot_dim].  d_cache NULL: nothing is appended (a layer that reads the rows another layer of equal
+ * kv_rank, rot_dim and rotation cached); only the queries' rotated parts are written. */
 int ktx_latattn_prep(const ktx_latattn_config* cfg, int T, const float* d_proj, int64_t ldp, int q_off, int c_off, const float* d_wn,
                      const double* d_inv_freq, const int32_t* d_pos, const int32_t* d_cache_loc, void* d_cache, float* d_q_out,
                      ktx_stream_t stream);
 
 /* out[t][h] = sum_j w_j c_j over the keys j in the window of token t, w = softmax over {scale q[t][h] . row_j} u {sink[h]} with the
- * sink's weight dropped (it has no value).  q fp32 [T][heads][kv_rank + rot_dim]; out [T][heads][kv_rank] of out_dtype.
+ * sink's weight dropped (it has no value; d_sink NULL: an ordinary softmax over the keys).  q fp32 [T][heads][kv_rank + rot_dim]; out [T][heads][kv_rank] of out_dtype.
  * nsplit workgroups share a token's keys: scratch fp32 [nsplit][T][heads][kv_rank + 2] when nsplit > 1. */
 int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, const void* d_cache, const int32_t* d_tok_req,
                         const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices, const float* d_sink,

@@ -86,6 +86,8 @@ typedef struct ktx_swa_config {
   float scale;                        /* score = scale * (q . k) */
   int32_t window;                     /* position i sees j with 0 <= i - j < window; <= 0: no window */
   int32_t page_size, cache_dtype;     /* caches [rows][kv_heads][dim] and [rows][kv_heads][vdim] of KTX_SEQ_* */
+  int32_t keep_first;                 /* with a window: the first keep_first positions of a sequence stay visible to every later one */
+  int32_t bias_span;                  /* rows - 1 of the distance-bias table the attention calls take (distances beyond it read its last row) */
 } ktx_swa_config;
 
 /* Per token: rotate and norm q (times scale) -> q_out fp32 [T][heads][dim]; rotate and norm k, turn v -> cache rows cache_loc[t];
@@ -96,21 +98,37 @@ int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t 
                  const double* d_inv_freq, const double* d_v_inv_freq, const int32_t* d_pos, const int32_t* d_cache_loc, void* d_kcache,
                  void* d_vcache, float* d_q_out, float* d_vcs, ktx_stream_t stream);
 
-/* out[t][h] = turn_back(sum_j p_j v_j), p = softmax over {q[t][h] . k_j : j in the window of t} and, with sink (fp32 [heads]), one more
- * score sink[h] that has no value.  Vector-ALU form, any sizes and either cache type: one token x the query heads of one key head x
+/* The prep of the un-rotated form whose projections pass a short causal convolution over time: with u = proj[t] + bias (q | k | v, C =
+ * heads dim + kv_heads (dim + vdim) channels at column 0 of fp32 rows of stride ldp; bias fp32 [C] or NULL),
+ *   y[t][c] = sum_{j < taps} conv_w[c][j] u[t - taps + 1 + j][c]      (conv_w fp32 [C][taps], the last column multiplies the current token;
+ *             inputs before a request's first NEW token come from its slot of conv_state fp32 [slots][taps - 1][C] when pos0 > 0 and are
+ *             zero otherwise; taps <= 1: y = u, times conv_w when given)
+ *   q = y_q / sqrt(mean(y_q^2) + eps) * q_norm_w * scale over ALL heads dim entries at once (q_norm_w fp32 [heads dim] or NULL: no norm),
+ *   k likewise with k_norm_w over kv_heads dim entries; q -> q_out fp32 [T][heads][dim], k and v = y_v -> cache rows cache_loc[t].
+ * Then (second launch) conv_state[slot[b]] = the last taps - 1 inputs u of request b.  cfg: rot_dims = 0, rot_values = 0; taps <= 16. */
+int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
+                      const float* d_conv_w, const float* d_q_norm_w, const float* d_k_norm_w, const int32_t* d_q_indptr,
+                      const int32_t* d_pos0, const int32_t* d_slot, const int32_t* d_tok_req, float* d_conv_state,
+                      const int32_t* d_cache_loc, void* d_kcache, void* d_vcache, float* d_q_out, ktx_stream_t stream);
+
+/* out[t][h] = turn_back(sum_j p_j v_j), p = softmax over {q[t][h] . k_j + dist_bias[min(i - j, bias_span)][h] : j visible to t at
+ * position i: j <= i and (i - j < window or j < keep_first)} and, with sink (fp32 [heads]), one more score sink[h] that has no value.
+ * dist_bias: fp32 [bias_span + 1][heads] or NULL (not scaled: scale is folded into q).  Vector-ALU form, any sizes and either cache type: one token x the query heads of one key head x
  * one key range per workgroup; nsplit key ranges leave partial sums in scratch fp32 [nsplit][T][heads][vdim + 2], merged afterwards.
  * out [T][heads * vdim] of out_dtype. */
 int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const void* d_kcache, const void* d_vcache,
                     const int32_t* d_tok_req, const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices,
-                    const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream);
+                    const float* d_sink, const float* d_dist_bias, const float* d_vcs, int nsplit, float* d_scratch, void* d_out,
+                    int out_dtype, ktx_stream_t stream);
 
 /* The same operator on the matrix cores for prompts, portions and decode steps: the (token, head) pairs of a request that share a key
  * head are the rows of one query matrix; workgroups of 64 rows walk 32-key tiles, bf16 MFMA for q . k and weights x values, scores /
- * mask / softmax in fp32.  Eligible: bf16 caches, dim a multiple of 32 up to 256, vdim 32 / 64 / 96 / 128 / 256. */
+ * mask / softmax in fp32.  Eligible: bf16 caches, dim a multiple of 32 up to 256, vdim a multiple of 16 up to 128, or 256. */
 int ktx_swa_mfma_eligible(const ktx_swa_config* cfg);
 int ktx_swa_mfma(const ktx_swa_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache, const void* d_vcache,
                  const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,
-                 const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream);
+                 const float* d_sink, const float* d_dist_bias, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype,
+                 ktx_stream_t stream);
 
 /* ---- selective scan --------------------------------------------------------------------------------------------------------------- */
 typedef struct ktx_ssm_config {

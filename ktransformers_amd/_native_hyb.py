@@ -16,10 +16,16 @@ class _DeltaConfig(C.Structure):     # include/ktx_hyb.h: ktx_delta_config
                 ("unit_eps", C.c_float)]
 
 
+class _PostNormArgs(C.Structure):    # include/ktx_hyb.h: ktx_postnorm_args
+    _fields_ = [("y", C.c_void_p), ("ldy", C.c_int64), ("ybias", C.c_void_p), ("alpha", C.c_float), ("w", C.c_void_p), ("b", C.c_void_p),
+                ("eps", C.c_float), ("stack", C.c_void_p), ("stack_stride", C.c_int64), ("level", C.c_int32), ("dwa", C.c_void_p),
+                ("out_lp", C.c_void_p), ("out_dtype", C.c_int32)]
+
+
 class _LatAttnConfig(C.Structure):   # include/ktx_hyb.h: ktx_latattn_config
     _fields_ = [("heads", C.c_int32), ("dim", C.c_int32), ("rot_dim", C.c_int32), ("vdim", C.c_int32), ("kv_rank", C.c_int32),
                 ("rot_dims", C.c_int32), ("scale", C.c_float), ("window", C.c_int32), ("eps", C.c_float), ("page_size", C.c_int32),
-                ("cache_dtype", C.c_int32)]
+                ("cache_dtype", C.c_int32), ("rot_half", C.c_int32)]
 
 
 _P, _I, _L, _F = C.c_void_p, C.c_int, C.c_int64, C.c_float
@@ -30,6 +36,9 @@ lib.ktx_layer_norm.argtypes = [_I, _I, _P, _P, _P, _F, _P, _P, _I, _P]
 lib.ktx_gated_norm_add.argtypes = [_I, _I, _P, _L, _P, _P, _P, _P, _I, _P, _L, _P, _P, _P, _F, _P, _P, _P, _F, _P, _I, _P]
 lib.ktx_poly_norm.argtypes = [_I, _I, _P, _L, _P, _P, _F, _P, _I, _P]
 lib.ktx_silu_mul_rows.argtypes = [_I, _I, _P, _L, _P, _I, _P]
+lib.ktx_postnorm_mix.argtypes = [_I, _I, _P, _P, C.POINTER(_PostNormArgs), _P]
+lib.ktx_glu_clamp_rows.argtypes = [_I, _I, _P, _L, _F, _F, _F, _P, _I, _P]
+lib.ktx_sigmoid_gate_rows.argtypes = [_I, _I, _P, _I, _P, _L, _P, _I, _P]
 lib.ktx_head_gate_norm.argtypes = [_I, _I, _I, _F, _P, _P, _L, _P, _I, _I, _P, _I, _P]
 lib.ktx_delta_prep.argtypes = [C.POINTER(_DeltaConfig), _I, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P]
 lib.ktx_delta_forward.argtypes = [C.POINTER(_DeltaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P]
@@ -142,6 +151,52 @@ def silu_mul_rows(gu: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
     return out
 
 
+def postnorm_mix(x_in: torch.Tensor, x_out: torch.Tensor, w: torch.Tensor, b: torch.Tensor | None, eps: float, alpha: float = 1.0,
+                 y: torch.Tensor | None = None, ybias: torch.Tensor | None = None, stack: torch.Tensor | None = None, level: int = 0,
+                 dwa: torch.Tensor | None = None, lp_dtype=None):
+    """One launch (ktx_postnorm_mix): v = layer_norm(alpha * x_in + y + ybias; w, b, eps); with stack fp32 [levels, T, W], level `level`
+    receives v, and with dwa fp32 [level + 1] the rows handed on are sum_j dwa[j] * stack[j]; x_out fp32 [T, W] (may be x_in) receives
+    them.  Returns a copy of x_out in lp_dtype when that is given (what the following products read), else x_out."""
+    _f32(x_in, "postnorm_mix x_in"), _f32(x_out, "postnorm_mix x_out"), _f32(w, "postnorm_mix w"), _f32(b, "postnorm_mix b")
+    _f32(ybias, "postnorm_mix ybias"), _f32(stack, "postnorm_mix stack"), _f32(dwa, "postnorm_mix dwa")
+    T, W = x_in.shape
+    yp, ldy = _rows_f32(y, "postnorm_mix y")
+    if tuple(x_out.shape) != (T, W) or w.numel() != W or (b is not None and b.numel() != W) or (ybias is not None and ybias.numel() != W) or \
+            (y is not None and tuple(y.shape) != (T, W)):
+        raise KtxError("postnorm_mix: shapes do not fit")
+    if stack is not None and (stack.dim() != 3 or tuple(stack.shape[1:]) != (T, W) or not 0 <= level < stack.shape[0]):
+        raise KtxError("postnorm_mix: stack must be [levels, T, W] with level inside")
+    if dwa is not None and (stack is None or dwa.numel() != level + 1):
+        raise KtxError("postnorm_mix: the average takes level + 1 weights and the stack")
+    lp = torch.empty((T, W), dtype=lp_dtype, device=x_in.device) if lp_dtype is not None and lp_dtype != torch.float32 else None
+    a = _PostNormArgs(yp, ldy, _ptr(ybias), float(alpha), w.data_ptr(), _ptr(b), float(eps), _ptr(stack),
+                      stack.stride(0) if stack is not None else 0, int(level), _ptr(dwa), _ptr(lp), SEQ_DTYPE[lp.dtype] if lp is not None else 0)
+    check(lib.ktx_postnorm_mix(T, W, x_in.data_ptr(), x_out.data_ptr(), C.byref(a), _stream_ptr(x_in.device)))
+    return x_out if lp is None else lp
+
+
+def glu_clamp_rows(gu: torch.Tensor, limit: float | None, slope: float = 1.0, up_shift: float = 0.0, out_dtype=torch.float32) -> torch.Tensor:
+    """[R, 2F] (gate | up) -> g * sigmoid(slope * g) * (u + up_shift), g = min(gate, limit), u = clamp(up, -limit, limit); [R, F]
+    (ktx_glu_clamp_rows; limit None: neither is bounded)."""
+    p, ld = _rows_f32(gu, "glu_clamp_rows")
+    R, F = gu.shape[0], gu.shape[1] // 2
+    out = torch.empty((R, F), dtype=out_dtype, device=gu.device)
+    check(lib.ktx_glu_clamp_rows(R, F, p, ld, float("inf") if limit is None else float(limit), float(slope), float(up_shift),
+                                 out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(gu.device)))
+    return out
+
+
+def sigmoid_gate_rows(o: torch.Tensor, gate: torch.Tensor, out_dtype=torch.float32) -> torch.Tensor:
+    """o [R, N] (contiguous, fp32 | bf16) * sigmoid(gate), gate fp32 rows [R, N] (a column slice is fine) -> [R, N] of out_dtype."""
+    gp, ldg = _rows_f32(gate, "sigmoid_gate_rows gate")
+    if o.dim() != 2 or not o.is_contiguous() or o.dtype not in SEQ_DTYPE or tuple(gate.shape) != tuple(o.shape):
+        raise KtxError("sigmoid_gate_rows: o must be contiguous rows of the gate's shape")
+    out = torch.empty(o.shape, dtype=out_dtype, device=o.device)
+    check(lib.ktx_sigmoid_gate_rows(o.shape[0], o.shape[1], o.data_ptr(), SEQ_DTYPE[o.dtype], gp, ldg, out.data_ptr(), SEQ_DTYPE[out_dtype],
+                                    _stream_ptr(o.device)))
+    return out
+
+
 def head_gate_norm(o: torch.Tensor, gate: torch.Tensor, w: torch.Tensor, heads: int, vdim: int, eps: float, w_per_head: bool, act: str,
                    out_dtype=torch.float32) -> torch.Tensor:
     _f32(o, "head_gate_norm o"), _f32(w, "head_gate_norm w")
@@ -190,22 +245,27 @@ def delta_forward(cfg: _DeltaConfig, qkv: torch.Tensor, gb: torch.Tensor, batch,
 
 
 def latattn_config(heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, rot_dims: int, scale: float, window: int, eps: float,
-                   page_size: int, cache_dtype) -> _LatAttnConfig:
+                   page_size: int, cache_dtype, rot_half: bool = False) -> _LatAttnConfig:
     return _LatAttnConfig(heads, dim, rot_dim, vdim, kv_rank, int(rot_dims), float(scale), int(window), float(eps), int(page_size),
-                          SEQ_DTYPE[cache_dtype])
+                          SEQ_DTYPE[cache_dtype], 1 if rot_half else 0)
 
 
-def latattn_prep(cfg: _LatAttnConfig, proj: torch.Tensor, q_off: int, c_off: int, wn: torch.Tensor, inv_freq: torch.Tensor,
-                 positions: torch.Tensor, cache_loc: torch.Tensor, cache: torch.Tensor, q_out: torch.Tensor) -> None:
+def latattn_prep(cfg: _LatAttnConfig, proj: torch.Tensor, q_off: int, c_off: int, wn: torch.Tensor | None, inv_freq: torch.Tensor,
+                 positions: torch.Tensor, cache_loc: torch.Tensor, cache: torch.Tensor | None, q_out: torch.Tensor) -> None:
+    """cache None (and wn None, c_off ignored): only the queries' rotated parts are written — the layer reads latent rows that another
+    layer appended."""
     pp, ldp = _rows_f32(proj, "latattn_prep proj")
     _f32(wn, "latattn_prep wn"), _f32(q_out, "latattn_prep q_out"), _i32(positions, "positions"), _i32(cache_loc, "cache_loc")
     _seq_dev(inv_freq, torch.float64, "latattn_prep inv_freq")
     T, E = proj.shape[0], cfg.kv_rank + cfg.rot_dim
-    if positions.numel() != T or cache_loc.numel() != T or cache.shape[-1] != E or q_out.numel() != T * cfg.heads * E or \
-            inv_freq.numel() != cfg.rot_dims // 2 or wn.numel() != cfg.kv_rank or not cache.is_contiguous():
+    if positions.numel() != T or cache_loc.numel() != T or q_out.numel() != T * cfg.heads * E or inv_freq.numel() != cfg.rot_dims // 2 or \
+            proj.shape[1] < q_off + cfg.heads * (cfg.dim + cfg.rot_dim):
         raise KtxError("latattn_prep: shapes do not fit")
-    check(lib.ktx_latattn_prep(C.byref(cfg), T, pp, ldp, q_off, c_off, wn.data_ptr(), inv_freq.data_ptr(), positions.data_ptr(),
-                               cache_loc.data_ptr(), cache.data_ptr(), q_out.data_ptr(), _stream_ptr(proj.device)))
+    if cache is not None and (cache.shape[-1] != E or wn is None or wn.numel() != cfg.kv_rank or not cache.is_contiguous()
+                              or proj.shape[1] < c_off + E or int(cache.numel()) // E <= 0):
+        raise KtxError("latattn_prep: cache / latent norm do not fit")
+    check(lib.ktx_latattn_prep(C.byref(cfg), T, pp, ldp, q_off, c_off, _ptr(wn), inv_freq.data_ptr(), positions.data_ptr(),
+                               cache_loc.data_ptr(), _ptr(cache), q_out.data_ptr(), _stream_ptr(proj.device)))
 
 
 def latattn_forward(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, batch, sink: torch.Tensor, nsplit: int = 1,
@@ -216,7 +276,7 @@ def latattn_forward(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, b
     out = torch.empty((T, cfg.heads * L), dtype=out_dtype, device=q.device)
     scratch = torch.empty((nsplit, T, cfg.heads, L + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
     check(lib.ktx_latattn_forward(C.byref(cfg), T, q.data_ptr(), cache.data_ptr(), batch.tok_req.data_ptr(), batch.positions.data_ptr(),
-                                  batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), sink.data_ptr(), int(nsplit), _ptr(scratch),
+                                  batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), _ptr(sink), int(nsplit), _ptr(scratch),
                                   out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
     return out
 
@@ -233,7 +293,7 @@ def latattn_mfma(cfg: _LatAttnConfig, q: torch.Tensor, cache: torch.Tensor, batc
     out = torch.empty((T, cfg.heads * L), dtype=out_dtype, device=q.device)
     scratch = torch.empty((nsplit, T, cfg.heads, L + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
     check(lib.ktx_latattn_mfma(C.byref(cfg), batch.B, T, int(batch.max_q_len), q.data_ptr(), cache.data_ptr(), batch.q_indptr.data_ptr(),
-                               batch.pos0.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), sink.data_ptr(),
+                               batch.pos0.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), _ptr(sink),
                                int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
     return out
 

@@ -95,13 +95,16 @@ def embed_sinpos(tokens: torch.Tensor, positions: torch.Tensor, embed: torch.Ten
     return x
 
 
-def embed_rows(tokens: torch.Tensor, embed: torch.Tensor) -> torch.Tensor:
-    """tokens int32 [T]; embed [vocab, width] bf16 | fp32 -> the table rows as fp32 [T, width] (ktx_embed_sinpos without positions)."""
+def embed_rows(tokens: torch.Tensor, embed: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """tokens int32 [T]; embed [vocab, width] bf16 | fp32 -> the table rows as fp32 [T, width] (ktx_embed_sinpos without positions);
+    `out`: a contiguous fp32 [T, width] tensor to write them into."""
     _seq_dev(tokens, torch.int32, "embed_rows tokens"), _seq_dev(embed, None, "embed_rows embed")
     if embed.dtype not in SEQ_DTYPE:
         raise KtxError("embed_rows: element type does not fit")
     T, (vocab, width) = tokens.numel(), embed.shape
-    x = torch.empty((T, width), dtype=torch.float32, device=tokens.device)
+    if out is not None and (tuple(_seq_dev(out, torch.float32, "embed_rows out").shape) != (T, width)):
+        raise KtxError("embed_rows: out must be fp32 [T, width]")
+    x = out if out is not None else torch.empty((T, width), dtype=torch.float32, device=tokens.device)
     check(lib.ktx_embed_sinpos(T, width, vocab, tokens.data_ptr(), None, embed.data_ptr(), SEQ_DTYPE[embed.dtype], None, x.data_ptr(),
                                _stream_ptr(x.device)))
     return x

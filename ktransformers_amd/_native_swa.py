@@ -22,7 +22,8 @@ class _ResidArgs(C.Structure):       # include/ktx_swa.h: ktx_resid_args
 
 class _SwaConfig(C.Structure):       # include/ktx_swa.h: ktx_swa_config
     _fields_ = [("heads", _I32), ("kv_heads", _I32), ("dim", _I32), ("vdim", _I32), ("rot_dims", _I32), ("rot_values", _I32),
-                ("qk_norm", _I32), ("eps", _F), ("scale", _F), ("window", _I32), ("page_size", _I32), ("cache_dtype", _I32)]
+                ("qk_norm", _I32), ("eps", _F), ("scale", _F), ("window", _I32), ("page_size", _I32), ("cache_dtype", _I32),
+                ("keep_first", _I32), ("bias_span", _I32)]
 
 
 class _SsmConfig(C.Structure):       # include/ktx_swa.h: ktx_ssm_config
@@ -35,9 +36,10 @@ lib.ktx_resid_norm.argtypes = [_I, _I, _P, C.POINTER(_ResidArgs), _P]
 lib.ktx_input_conv.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P]
 lib.ktx_rows_mul_lookup.argtypes = [_I, _I, _P, _L, _P, _I, _L, _I, _P, _P, _I, _P]
 lib.ktx_swa_prep.argtypes = [C.POINTER(_SwaConfig), _I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]
-lib.ktx_swa_forward.argtypes = [C.POINTER(_SwaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
+lib.ktx_swa_conv_prep.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _P, _L] + [_P] * 14
+lib.ktx_swa_forward.argtypes = [C.POINTER(_SwaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_swa_mfma_eligible.argtypes = [C.POINTER(_SwaConfig)]
-lib.ktx_swa_mfma.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
+lib.ktx_swa_mfma.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_ssm_conv.argtypes = [C.POINTER(_SsmConfig), _I, _I, _P, _P, _P, _P, _P, _L, _I, _P, _P, _P, _P, _P]
 lib.ktx_ssm_scan.argtypes = [C.POINTER(_SsmConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _L, _P, _L, _P, _P, _P, _P, _L, _I, _I, _P, _P, _P,
                              _I, _P]
@@ -169,9 +171,39 @@ def rows_mul_lookup(a: torch.Tensor, table: torch.Tensor, col0: int, tokens: tor
 
 
 def swa_config(heads: int, kv_heads: int, dim: int, vdim: int, rot_dims: int, rot_values: bool, qk_norm: bool, eps: float, scale: float,
-               window: int, page_size: int, cache_dtype) -> _SwaConfig:
+               window: int, page_size: int, cache_dtype, keep_first: int = 0, bias_span: int = 0) -> _SwaConfig:
+    """keep_first: with a window, the sequence's first positions that stay visible; bias_span: rows - 1 of the distance-bias table the
+    attention calls are given (`dist_bias`)."""
     return _SwaConfig(heads, kv_heads, dim, vdim, int(rot_dims), int(bool(rot_values)), int(bool(qk_norm)), float(eps), float(scale),
-                      int(window), int(page_size), SEQ_DTYPE[cache_dtype])
+                      int(window), int(page_size), SEQ_DTYPE[cache_dtype], int(keep_first), int(bias_span))
+
+
+def swa_conv_prep(cfg: _SwaConfig, proj: torch.Tensor, bias: torch.Tensor | None, conv_w: torch.Tensor | None, q_norm_w: torch.Tensor | None,
+                  k_norm_w: torch.Tensor | None, batch, conv_state: torch.Tensor | None, kcache: torch.Tensor, vcache: torch.Tensor) -> torch.Tensor:
+    """The un-rotated prep with a causal convolution over time behind the projections and RMS norms over the whole q and k projections
+    (ktx_swa_conv_prep): proj fp32 [T, >= C] with q | k | v at column 0 -> q fp32 [T, heads * dim] (normed, scaled); key and value rows
+    are appended, the convolution's state slots move on.  conv_w fp32 [C, taps] or None."""
+    pp, ldp = _rows_f32(proj, "swa_conv_prep proj")
+    for t_, what in ((bias, "bias"), (conv_w, "conv_w"), (q_norm_w, "q_norm_w"), (k_norm_w, "k_norm_w"), (conv_state, "conv_state")):
+        _f32(t_, "swa_conv_prep " + what)
+    T = proj.shape[0]
+    nq, nk, nv = cfg.heads * cfg.dim, cfg.kv_heads * cfg.dim, cfg.kv_heads * cfg.vdim
+    Cn = nq + nk + nv
+    taps = int(conv_w.shape[1]) if conv_w is not None else 0
+    if batch.positions.numel() != T or batch.cache_loc.numel() != T or proj.shape[1] < Cn or \
+            tuple(kcache.shape[1:]) != (cfg.kv_heads, cfg.dim) or tuple(vcache.shape[1:]) != (cfg.kv_heads, cfg.vdim) or \
+            not kcache.is_contiguous() or not vcache.is_contiguous() or kcache.dtype != vcache.dtype or \
+            SEQ_DTYPE.get(kcache.dtype) != cfg.cache_dtype or (bias is not None and bias.numel() != Cn) or \
+            (conv_w is not None and tuple(conv_w.shape) != (Cn, taps)) or (q_norm_w is not None and q_norm_w.numel() != nq) or \
+            (k_norm_w is not None and k_norm_w.numel() != nk) or \
+            (taps > 1 and (conv_state is None or tuple(conv_state.shape[1:]) != (taps - 1, Cn))):
+        raise KtxError("swa_conv_prep: shapes do not fit")
+    q = torch.empty((T, nq), dtype=torch.float32, device=proj.device)
+    check(lib.ktx_swa_conv_prep(C.byref(cfg), batch.B, T, taps, pp, ldp, _ptr(bias), _ptr(conv_w), _ptr(q_norm_w), _ptr(k_norm_w),
+                                batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(), batch.tok_req.data_ptr(),
+                                _ptr(conv_state), batch.cache_loc.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), q.data_ptr(),
+                                _stream_ptr(proj.device)))
+    return q
 
 
 def swa_prep(cfg: _SwaConfig, proj: torch.Tensor, q_off: int, k_off: int, v_off: int, inv_freq: torch.Tensor | None,
@@ -196,16 +228,23 @@ def swa_prep(cfg: _SwaConfig, proj: torch.Tensor, q_off: int, k_off: int, v_off:
     return q, vcs
 
 
+def _dist_bias_ok(cfg: _SwaConfig, dist_bias) -> None:
+    _f32(dist_bias, "dist_bias")
+    if dist_bias is not None and tuple(dist_bias.shape) != (cfg.bias_span + 1, cfg.heads):
+        raise KtxError(f"dist_bias: expected fp32 [{cfg.bias_span + 1}, {cfg.heads}], got {tuple(dist_bias.shape)}")
+
+
 def swa_forward(cfg: _SwaConfig, q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, batch, sink: torch.Tensor | None,
-                vcs: torch.Tensor | None, nsplit: int = 1, out_dtype=torch.float32) -> torch.Tensor:
-    """The vector-ALU form (ktx_swa_forward) -> [T, heads * vdim] of out_dtype."""
-    _f32(q, "swa_forward q"), _f32(sink, "swa_forward sink"), _f32(vcs, "swa_forward vcs")
+                vcs: torch.Tensor | None, nsplit: int = 1, out_dtype=torch.float32, dist_bias: torch.Tensor | None = None) -> torch.Tensor:
+    """The vector-ALU form (ktx_swa_forward) -> [T, heads * vdim] of out_dtype.  dist_bias fp32 [cfg.bias_span + 1, heads]: added to the
+    score by distance (the last row serves every larger distance)."""
+    _f32(q, "swa_forward q"), _f32(sink, "swa_forward sink"), _f32(vcs, "swa_forward vcs"), _dist_bias_ok(cfg, dist_bias)
     T = q.shape[0]
     out = torch.empty((T, cfg.heads * cfg.vdim), dtype=out_dtype, device=q.device)
     scratch = torch.empty((nsplit, T, cfg.heads, cfg.vdim + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
     check(lib.ktx_swa_forward(C.byref(cfg), T, q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), batch.tok_req.data_ptr(),
-                              batch.positions.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), _ptr(sink), _ptr(vcs),
-                              int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
+                              batch.positions.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(), _ptr(sink),
+                              _ptr(dist_bias), _ptr(vcs), int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
     return out
 
 
@@ -214,15 +253,16 @@ def swa_mfma_eligible(cfg: _SwaConfig) -> bool:
 
 
 def swa_mfma(cfg: _SwaConfig, q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, batch, sink: torch.Tensor | None,
-             vcs: torch.Tensor | None, nsplit: int = 1, out_dtype=torch.bfloat16) -> torch.Tensor:
+             vcs: torch.Tensor | None, nsplit: int = 1, out_dtype=torch.bfloat16, dist_bias: torch.Tensor | None = None) -> torch.Tensor:
     """The matrix-core form, prompts and decode steps (ktx_swa_mfma) -> [T, heads * vdim] of out_dtype."""
-    _f32(q, "swa_mfma q"), _f32(sink, "swa_mfma sink"), _f32(vcs, "swa_mfma vcs")
+    _f32(q, "swa_mfma q"), _f32(sink, "swa_mfma sink"), _f32(vcs, "swa_mfma vcs"), _dist_bias_ok(cfg, dist_bias)
     T = q.shape[0]
     out = torch.empty((T, cfg.heads * cfg.vdim), dtype=out_dtype, device=q.device)
     scratch = torch.empty((nsplit, T, cfg.heads, cfg.vdim + 2), dtype=torch.float32, device=q.device) if nsplit > 1 else None
     check(lib.ktx_swa_mfma(C.byref(cfg), batch.B, T, int(batch.max_q_len), q.data_ptr(), kcache.data_ptr(), vcache.data_ptr(),
                            batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.page_indptr.data_ptr(), batch.page_indices.data_ptr(),
-                           _ptr(sink), _ptr(vcs), int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(q.device)))
+                           _ptr(sink), _ptr(dist_bias), _ptr(vcs), int(nsplit), _ptr(scratch), out.data_ptr(), SEQ_DTYPE[out_dtype],
+                           _stream_ptr(q.device)))
     return out
 
 

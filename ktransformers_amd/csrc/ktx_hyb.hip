@@ -107,6 +107,53 @@ __global__ void __launch_bounds__(256) gated_norm_add_kernel(int W, const float*
   for (int e = tid; e < W; e += 256) st_elem(nout, (size_t)t * W + e, (zrow[e] - mean2) * r2 * nw[e] + (nb ? nb[e] : 0.f));
 }
 
+// v = layer_norm(alpha * x + y + ybias); with a stack: level `level` of it receives v, and with dwa the row handed on is the weighted
+// sum of levels 0 .. level.  The row lives in LDS between the passes; every level's entry is requested before the sum is formed.
+template <typename OT>
+__global__ void __launch_bounds__(256) postnorm_mix_kernel(int W, const float* __restrict__ xin, float* __restrict__ xout,
+                                                           ktx_postnorm_args a, OT* __restrict__ lp) {
+  extern __shared__ float zrow[];
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const size_t ro = (size_t)t * W;
+  float s = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    float z = a.alpha * xin[ro + e];
+    if (a.y) z += a.y[(size_t)t * a.ldy + e];
+    if (a.ybias) z += a.ybias[e];
+    zrow[e] = z;
+    s += z;
+  }
+  const float mean = block_sum256(s, red) / (float)W;
+  float q = 0.f;
+  for (int e = tid; e < W; e += 256) {
+    const float d = zrow[e] - mean;
+    q += d * d;
+  }
+  const float r = 1.0f / sqrtf(block_sum256(q, red) / (float)W + a.eps);
+  const int lv = a.level;
+  for (int e = tid; e < W; e += 256) {
+    float v = (zrow[e] - mean) * r * a.w[e] + (a.b ? a.b[e] : 0.f);
+    if (a.stack) {
+      a.stack[(size_t)lv * a.stack_stride + ro + e] = v;
+      if (a.dwa) {
+        float m = a.dwa[lv] * v;
+        for (int j0 = 0; j0 < lv; j0 += 8) {
+          float part[8];
+#pragma unroll
+          for (int i = 0; i < 8; i++) part[i] = j0 + i < lv ? a.stack[(size_t)(j0 + i) * a.stack_stride + ro + e] : 0.f;
+#pragma unroll
+          for (int i = 0; i < 8; i++)
+            if (j0 + i < lv) m += a.dwa[j0 + i] * part[i];
+        }
+        v = m;
+      }
+    }
+    xout[ro + e] = v;
+    if (lp) st_elem(lp, ro + e, v);
+  }
+}
+
 template <typename OT>
 __global__ void __launch_bounds__(256) poly_norm_kernel(int F, const float* __restrict__ zin, int64_t ldz, const float* __restrict__ bias,
                                                         const float* __restrict__ coef, float eps, OT* __restrict__ out) {
@@ -128,6 +175,27 @@ __global__ void __launch_bounds__(256) poly_norm_kernel(int F, const float* __re
     const float z = a[e] + (bias ? bias[e] : 0.f), z2 = z * z;
     st_elem(out, (size_t)t * F + e, ((z * r1 + z2 * r2) + z2 * z * r3) + c3);
   }
+}
+
+// out[r][f] = g * sigmoid(slope * g) * (u + up_shift), g = min(in[r][f], limit), u = clamp(in[r][F + f], -limit, limit)
+template <typename OT>
+__global__ void __launch_bounds__(256) glu_clamp_rows_kernel(size_t n, int F, const float* __restrict__ in, int64_t ldi, float limit,
+                                                             float slope, float up_shift, OT* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  const size_t r = i / F;
+  const int f = (int)(i % F);
+  const float g = fminf(in[r * ldi + f], limit), u = fminf(fmaxf(in[r * ldi + F + f], -limit), limit);
+  st_elem(out, i, g * sigmoid_f32(slope * g) * (u + up_shift));
+}
+
+// out[r][c] = o[r][c] * sigmoid(gate[r][c])
+template <typename IT, typename OT>
+__global__ void __launch_bounds__(256) sigmoid_gate_rows_kernel(size_t n, int N, const IT* __restrict__ o, const float* __restrict__ gate,
+                                                                int64_t ldg, OT* __restrict__ out) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= n) return;
+  st_elem(out, i, ld_elem(o, i) * sigmoid_f32(gate[(i / N) * ldg + i % N]));
 }
 
 template <typename OT>
@@ -378,20 +446,31 @@ __global__ void __launch_bounds__(256) latattn_prep_kernel(ktx_latattn_config c,
     cs[i] = (float)cos(a);
     cs[NP + i] = (float)sin(a);
   }
-  const float* lat = proj + (size_t)t * ldp + c_off;
-  float s = 0.f;
-  for (int e = tid; e < L; e += 256) s += lat[e] * lat[e];
-  const float r = 1.0f / sqrtf(block_sum256(s, red) / (float)L + c.eps);      // (its barriers also publish cs)
-  KT* row = cache + (size_t)cache_loc[t] * E;
-  for (int e = tid; e < L; e += 256) st_elem(row, e, lat[e] * r * wn[e]);
-  // rotated parts: entry j of a rotated vector; j < rot_dims turns with its partner
+  // rotated parts: entry j of a rotated vector; j < rot_dims turns with its partner — its neighbour (pairs 2i, 2i + 1), or, in the
+  // half layout, the entry rot_dims / 2 further on (pairs i, i + rot_dims / 2)
+  const bool half = c.rot_half != 0;
   auto turned = [&](const float* v, int j) -> float {
     if (j >= 2 * NP) return v[j];
+    if (half) {
+      const int i = j < NP ? j : j - NP;
+      const float a = v[i], bb = v[i + NP];
+      return j < NP ? a * cs[i] - bb * cs[NP + i] : bb * cs[i] + a * cs[NP + i];
+    }
     const int i = j >> 1;
     const float a = v[2 * i], bb = v[2 * i + 1];
     return (j & 1) ? bb * cs[i] + a * cs[NP + i] : a * cs[i] - bb * cs[NP + i];
   };
-  for (int j = tid; j < R; j += 256) st_elem(row, L + j, turned(lat + L, j));
+  if (cache) {                               // (a layer that reads another layer's latent rows has none of its own to append)
+    const float* lat = proj + (size_t)t * ldp + c_off;
+    float s = 0.f;
+    for (int e = tid; e < L; e += 256) s += lat[e] * lat[e];
+    const float r = 1.0f / sqrtf(block_sum256(s, red) / (float)L + c.eps);      // (its barriers also publish cs)
+    KT* row = cache + (size_t)cache_loc[t] * E;
+    for (int e = tid; e < L; e += 256) st_elem(row, e, lat[e] * r * wn[e]);
+    for (int j = tid; j < R; j += 256) st_elem(row, L + j, turned(lat + L, j));
+  } else {
+    __syncthreads();
+  }
   const int D = c.dim;
   for (int e = tid; e < c.heads * R; e += 256) {
     const int h = e / R, j = e % R;
@@ -493,10 +572,14 @@ __global__ void __launch_bounds__(256) latattn_fwd_kernel(ktx_latattn_config c, 
       const int e = tid + i * 256;
       if (e < nout) {
         const int h = e / L, l = e % L;
-        const float sk = sink[h0 + h], m = mrow[h];
-        const float M = fmaxf(m, sk);
-        const float f = m == -INFINITY ? 0.f : expf(m - M);
-        st_elem(out, ((size_t)t * c.heads + h0 + h) * L + l, acc[i] * f / (lrow[h] * f + expf(sk - M)));
+        const float m = mrow[h];
+        if (sink) {
+          const float sk = sink[h0 + h], M = fmaxf(m, sk);
+          const float f = m == -INFINITY ? 0.f : expf(m - M);
+          st_elem(out, ((size_t)t * c.heads + h0 + h) * L + l, acc[i] * f / (lrow[h] * f + expf(sk - M)));
+        } else {
+          st_elem(out, ((size_t)t * c.heads + h0 + h) * L + l, lrow[h] > 0.f ? acc[i] / lrow[h] : 0.f);
+        }
       }
     }
     return;
@@ -520,7 +603,6 @@ __global__ void __launch_bounds__(256) latattn_merge_kernel(int T, int H, int L,
   extern __shared__ float mw[];            // [nsplit] maxima, then [nsplit] weights exp(m_z - M) (0 for an empty range)
   float* ws = mw + nsplit;
   const int t = blockIdx.x, h = blockIdx.y;
-  const float sk = sink[h];
   const size_t stride = (size_t)T * H * (L + 2);
   const float* base = scratch + ((size_t)t * H + h) * (L + 2);
   for (int z = threadIdx.x; z < nsplit; z += 256) {
@@ -528,14 +610,14 @@ __global__ void __launch_bounds__(256) latattn_merge_kernel(int T, int H, int L,
     ws[z] = base[z * stride + L + 1];
   }
   __syncthreads();
-  float M = sk;
+  float M = sink ? sink[h] : -INFINITY;
   for (int z = 0; z < nsplit; z++) M = fmaxf(M, mw[z]);
-  float den = expf(sk - M);
+  float den = sink ? expf(sink[h] - M) : 0.f;
   for (int z = 0; z < nsplit; z++) den += mw[z] == -INFINITY ? 0.f : ws[z] * expf(mw[z] - M);
   __syncthreads();
   for (int z = threadIdx.x; z < nsplit; z += 256) ws[z] = mw[z] == -INFINITY ? 0.f : expf(mw[z] - M);
   __syncthreads();
-  const float inv = 1.0f / den;
+  const float inv = den > 0.f ? 1.0f / den : 0.f;
   for (int l = threadIdx.x; l < L; l += 256) {
     float a = 0.f;
 #pragma unroll 4
@@ -692,9 +774,14 @@ __global__ void __launch_bounds__(256) latattn_mfma_kernel(ktx_latattn_config c,
     const int cr = rw0 + lq * 4 + r;
     const size_t grow = (size_t)t0 * H + cr;             // (token, head) row of q / out
     if (nsplit == 1) {
-      const float sk = sink[hrow[r]], M = fmaxf(mrun[r], sk);
-      const float f = mrun[r] == -INFINITY ? 0.f : expf(mrun[r] - M);
-      const float inv = f / (lrun[r] * f + expf(sk - M));
+      float inv;
+      if (sink) {
+        const float sk = sink[hrow[r]], M = fmaxf(mrun[r], sk);
+        const float f = mrun[r] == -INFINITY ? 0.f : expf(mrun[r] - M);
+        inv = f / (lrun[r] * f + expf(sk - M));
+      } else {
+        inv = lrun[r] > 0.f ? 1.0f / lrun[r] : 0.f;
+      }
 #pragma unroll
       for (int n = 0; n < NT; n++) st_elem(out, grow * L + n * 16 + l16, acc[n][r] * inv);
     } else {
@@ -1080,6 +1167,60 @@ int ktx_poly_norm(int T, int F, const float* d_z, int64_t ldz, const float* d_bi
   return 0;
 }
 
+int ktx_postnorm_mix(int T, int W, const float* d_x_in, float* d_x_out, const ktx_postnorm_args* a, ktx_stream_t stream) {
+  KTX_REQUIRE(a && T >= 0 && W > 0 && d_x_in && d_x_out && a->w && (a->out_lp == nullptr || a->out_dtype == KTX_SEQ_BF16 || a->out_dtype == KTX_SEQ_F32),
+              "ktx_postnorm_mix: T >= 0, W > 0, x, a norm weight");
+  KTX_REQUIRE(!a->y || a->ldy >= W, "ktx_postnorm_mix: ldy >= W");
+  KTX_REQUIRE(!a->stack || (a->level >= 0 && a->stack_stride >= (int64_t)T * W), "ktx_postnorm_mix: level >= 0, stack_stride >= T * W");
+  KTX_REQUIRE(!a->dwa || a->stack, "ktx_postnorm_mix: the average needs the stack");
+  KTX_REQUIRE((size_t)W * 4 <= 150 * 1024, "ktx_postnorm_mix: a row must fit the LDS");
+  if (T == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (a->out_lp && a->out_dtype == KTX_SEQ_BF16) {
+    KTX_HIP(ktx_set_max_lds((const void*)postnorm_mix_kernel<bf16_t>, 150 * 1024));
+    postnorm_mix_kernel<bf16_t><<<T, 256, (size_t)W * 4, st>>>(W, d_x_in, d_x_out, *a, (bf16_t*)a->out_lp);
+  } else {
+    KTX_HIP(ktx_set_max_lds((const void*)postnorm_mix_kernel<float>, 150 * 1024));
+    postnorm_mix_kernel<float><<<T, 256, (size_t)W * 4, st>>>(W, d_x_in, d_x_out, *a, (float*)a->out_lp);
+  }
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, void* d_out, int out_dtype,
+                       ktx_stream_t stream) {
+  KTX_REQUIRE(R >= 0 && F > 0 && d_in && d_out && dtype_ok(out_dtype) && ldi >= 2 * (int64_t)F && limit > 0.f, "ktx_glu_clamp_rows: arguments");
+  if (R == 0) return 0;
+  const size_t n = (size_t)R * F;
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == KTX_SEQ_F32)
+    glu_clamp_rows_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, (float*)d_out);
+  else
+    glu_clamp_rows_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, (bf16_t*)d_out);
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
+int ktx_sigmoid_gate_rows(int R, int N, const void* d_o, int o_dtype, const float* d_gate, int64_t ldg, void* d_out, int out_dtype,
+                          ktx_stream_t stream) {
+  KTX_REQUIRE(R >= 0 && N > 0 && d_o && d_gate && d_out && dtype_ok(o_dtype) && dtype_ok(out_dtype) && ldg >= N, "ktx_sigmoid_gate_rows: arguments");
+  if (R == 0) return 0;
+  const size_t n = (size_t)R * N;
+  const unsigned blocks = (unsigned)((n + 255) / 256);
+  hipStream_t st = (hipStream_t)stream;
+#define KTX_SG_GO(IT, OT) sigmoid_gate_rows_kernel<IT, OT><<<blocks, 256, 0, st>>>(n, N, (const IT*)d_o, d_gate, ldg, (OT*)d_out)
+  if (o_dtype == KTX_SEQ_F32) {
+    if (out_dtype == KTX_SEQ_F32) KTX_SG_GO(float, float);
+    else KTX_SG_GO(float, bf16_t);
+  } else {
+    if (out_dtype == KTX_SEQ_F32) KTX_SG_GO(bf16_t, float);
+    else KTX_SG_GO(bf16_t, bf16_t);
+  }
+#undef KTX_SG_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
 int ktx_silu_mul_rows(int R, int F, const float* d_in, int64_t ldi, void* d_out, int out_dtype, ktx_stream_t stream) {
   KTX_REQUIRE(R >= 0 && F > 0 && d_in && d_out && dtype_ok(out_dtype) && ldi >= 2 * (int64_t)F, "ktx_silu_mul_rows: arguments");
   if (R == 0) return 0;
@@ -1168,7 +1309,7 @@ int ktx_latattn_prep(const ktx_latattn_config* cfg, int T, const float* d_proj, 
                      const double* d_inv_freq, const int32_t* d_pos, const int32_t* d_cache_loc, void* d_cache, float* d_q_out,
                      ktx_stream_t stream) {
   if (latattn_check(cfg, "ktx_latattn_prep")) return -1;
-  KTX_REQUIRE(T >= 0 && d_proj && d_wn && (d_inv_freq || cfg->rot_dims == 0) && d_pos && d_cache_loc && d_cache && d_q_out,
+  KTX_REQUIRE(T >= 0 && d_proj && (d_inv_freq || cfg->rot_dims == 0) && d_pos && d_q_out && (!d_cache || (d_wn && d_cache_loc)),
               "ktx_latattn_prep: null pointer");
   if (T == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
@@ -1185,7 +1326,7 @@ int ktx_latattn_forward(const ktx_latattn_config* cfg, int T, const float* d_q, 
                         const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices, const float* d_sink,
                         int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
   if (latattn_check(cfg, "ktx_latattn_forward")) return -1;
-  KTX_REQUIRE(T >= 0 && d_q && d_cache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_sink && d_out && dtype_ok(out_dtype),
+  KTX_REQUIRE(T >= 0 && d_q && d_cache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_out && dtype_ok(out_dtype),
               "ktx_latattn_forward: null pointer");
   KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_latattn_forward: 1 <= nsplit <= 4096, scratch when > 1");
   if (T == 0) return 0;
@@ -1239,7 +1380,7 @@ int ktx_latattn_mfma(const ktx_latattn_config* cfg, int B, int T, int max_q_len,
                      const float* d_sink, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
   if (latattn_check(cfg, "ktx_latattn_mfma")) return -1;
   KTX_REQUIRE(ktx_latattn_mfma_eligible(cfg), "ktx_latattn_mfma: bf16 cache, kv_rank 64 / 128 / 256 / 512, rot_dim a multiple of 8 up to 128");
-  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_cache && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices && d_sink &&
+  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_cache && d_q_indptr && d_pos0 && d_page_indptr && d_page_indices &&
                   d_out && dtype_ok(out_dtype),
               "ktx_latattn_mfma: null pointer");
   KTX_REQUIRE(nsplit >= 1 && nsplit <= 4096 && (nsplit == 1 || d_scratch), "ktx_latattn_mfma: 1 <= nsplit <= 4096, scratch when > 1");

@@ -243,6 +243,85 @@ __global__ void __launch_bounds__(256) swa_prep_kernel(ktx_swa_config c, const f
   }
 }
 
+// The prep of an attention whose projections pass a short causal convolution over time and whose q and k are RMS-normed over the WHOLE
+// projection (all heads at once) with a weight: one workgroup per token, the convolved q | k | v row in LDS between the passes.
+// Input u[c] at relative token ii of the request: this step's projection (+ bias) for ii >= 0, the slot's state row taps - 1 + ii for
+// ii < 0 when the request has a past, zero otherwise.
+constexpr int CP_MAX_TAPS = 16;
+template <typename KT>
+__global__ void __launch_bounds__(256) swa_conv_prep_kernel(ktx_swa_config c, int taps, const float* __restrict__ proj, int64_t ldp,
+                                                            const float* __restrict__ bias, const float* __restrict__ cw,
+                                                            const float* __restrict__ qw, const float* __restrict__ kw,
+                                                            const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                            const int32_t* __restrict__ slot, const int32_t* __restrict__ tok_req,
+                                                            const float* __restrict__ conv_state, const int32_t* __restrict__ cache_loc,
+                                                            KT* __restrict__ kcache, KT* __restrict__ vcache, float* __restrict__ q_out) {
+  extern __shared__ float row[];           // [H * D | G * D | G * V]
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int nq = c.heads * c.dim, nk = c.kv_heads * c.dim, nv = c.kv_heads * c.vdim, C = nq + nk + nv;
+  const int b = tok_req[t], i = t - q_indptr[b];
+  const bool carried = pos0[b] > 0;
+  const float* st = conv_state ? conv_state + (size_t)slot[b] * (taps - 1) * C : nullptr;
+  float sq = 0.f, sk = 0.f;
+  for (int e = tid; e < C; e += 256) {
+    const float be = bias ? bias[e] : 0.f;
+    float y;
+    if (taps <= 1) {
+      y = (proj[(size_t)t * ldp + e] + be) * (cw ? cw[e] : 1.0f);
+    } else {
+      float u[CP_MAX_TAPS];
+#pragma unroll
+      for (int j = 0; j < CP_MAX_TAPS; j++) {
+        u[j] = 0.f;
+        if (j < taps) {
+          const int ii = i - (taps - 1) + j;
+          if (ii >= 0) u[j] = proj[(size_t)(t - (taps - 1) + j) * ldp + e] + be;
+          else if (carried) u[j] = st[(size_t)(taps - 1 + ii) * C + e];
+        }
+      }
+      y = 0.f;
+#pragma unroll
+      for (int j = 0; j < CP_MAX_TAPS; j++)
+        if (j < taps) y += cw[(size_t)e * taps + j] * u[j];
+    }
+    row[e] = y;
+    if (e < nq) sq += y * y;
+    else if (e < nq + nk) sk += y * y;
+  }
+  const float rq = qw ? 1.0f / sqrtf(block_sum256(sq, red) / (float)nq + c.eps) : 1.0f;
+  const float rk = kw ? 1.0f / sqrtf(block_sum256(sk, red) / (float)nk + c.eps) : 1.0f;
+  const size_t loc = (size_t)cache_loc[t];
+  for (int e = tid; e < C; e += 256) {      // (each thread re-reads only what it wrote)
+    const float y = row[e];
+    if (e < nq) q_out[(size_t)t * nq + e] = y * rq * (qw ? qw[e] : 1.0f) * c.scale;
+    else if (e < nq + nk) st_elem(kcache, loc * nk + (e - nq), y * rk * (kw ? kw[e - nq] : 1.0f));
+    else st_elem(vcache, loc * nv + (e - nq - nk), y);
+  }
+}
+
+// the state of a causal convolution over C channels moves on behind a step: the slot's rows become the last taps - 1 inputs (this step's
+// projections + bias; older ones from the old state when the request brought fewer).  thread = channel, rows oldest first
+__global__ void __launch_bounds__(256) conv_state_update_kernel(int C, int taps, const int32_t* __restrict__ q_indptr,
+                                                                const int32_t* __restrict__ pos0, const int32_t* __restrict__ slot,
+                                                                const float* __restrict__ proj, int64_t ldp, const float* __restrict__ bias,
+                                                                float* __restrict__ conv_state) {
+  const int b = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+  if (e >= C) return;
+  const int first = q_indptr[b], n = q_indptr[b + 1] - first;
+  if (n <= 0) return;
+  const bool carried = pos0[b] > 0;
+  const float be = bias ? bias[e] : 0.f;
+  float* st = conv_state + (size_t)slot[b] * (taps - 1) * C;
+  for (int j = 0; j < taps - 1; j++) {      // row j takes the input n - (taps - 1) + j; an old row it may need lies further on (j + n > j)
+    const int ii = n - (taps - 1) + j;
+    float v = 0.f;
+    if (ii >= 0) v = proj[(size_t)(first + ii) * ldp + e] + be;
+    else if (carried) v = st[(size_t)(j + n) * C + e];
+    st[(size_t)j * C + e] = v;
+  }
+}
+
 // attention of ONE token (blockIdx.x) x HG query heads of one key head (blockIdx.y) x one key range (blockIdx.z) on the vector ALUs:
 // tiles of KTN <= 64 keys and values staged in LDS as fp32; scores thread = (head, key); running maximum / sum per head by wavefronts;
 // outputs thread = (head, value entry) in registers.
@@ -252,8 +331,9 @@ __global__ void __launch_bounds__(256) swa_fwd_kernel(ktx_swa_config c, int T, i
                                                       const KT* __restrict__ kcache, const KT* __restrict__ vcache,
                                                       const int32_t* __restrict__ tok_req, const int32_t* __restrict__ pos,
                                                       const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_indices,
-                                                      const float* __restrict__ sink, const float* __restrict__ vcs, int nsplit,
-                                                      float* __restrict__ scratch, OT* __restrict__ out) {
+                                                      const float* __restrict__ sink, const float* __restrict__ dist_bias,
+                                                      const float* __restrict__ vcs, int nsplit, float* __restrict__ scratch,
+                                                      OT* __restrict__ out) {
   extern __shared__ float lds[];
   const int D = c.dim, V = c.vdim, DP = D + 1, VP = V + 1, G = c.kv_heads, HPG = c.heads / G;
   float* qs = lds;                         // [HG][D]
@@ -264,14 +344,17 @@ __global__ void __launch_bounds__(256) swa_fwd_kernel(ktx_swa_config c, int T, i
   float* lrow = mrow + HG;                 // [HG] running sum
   float* crow = lrow + HG;                 // [HG] correction of this tile
   int* rowidx = reinterpret_cast<int*>(crow + HG);   // [KTN]
+  int* jpos = rowidx + KTN;                          // [KTN] the keys' positions
   const int t = blockIdx.x, g = blockIdx.y / parts, part = blockIdx.y % parts, z = blockIdx.z;
   const int h0 = g * HPG + part * HG;
   const int nh = min(HG, HPG - part * HG);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int p = pos[t], b = tok_req[t];
   const int jlo = c.window > 0 ? max(0, p - c.window + 1) : 0, jhi = p + 1;
-  const int per = (jhi - jlo + nsplit - 1) / nsplit;
-  const int j0 = jlo + z * per, j1 = min(jhi, j0 + per);
+  // the keys the token sees, as one list: the kept first positions that lie in front of the window, then the window
+  const int nfront = min(c.keep_first, jlo), nvis = nfront + (jhi - jlo);
+  const int per = (nvis + nsplit - 1) / nsplit;
+  const int j0 = z * per, j1 = min(nvis, j0 + per);
   for (int e = tid; e < nh * D; e += 256) qs[e] = q[((size_t)t * c.heads + h0) * D + e];
   for (int h = tid; h < HG; h += 256) {
     mrow[h] = -INFINITY;
@@ -286,8 +369,9 @@ __global__ void __launch_bounds__(256) swa_fwd_kernel(ktx_swa_config c, int T, i
     const int nk = min(KTN, j1 - jt);
     __syncthreads();
     if (tid < nk) {
-      const int j = jt + tid;
+      const int u = jt + tid, j = u < nfront ? u : jlo + (u - nfront);
       rowidx[tid] = pages[j / c.page_size] * c.page_size + j % c.page_size;
+      jpos[tid] = j;
     }
     __syncthreads();
     for (int e = tid; e < nk * D; e += 256) {
@@ -306,6 +390,7 @@ __global__ void __launch_bounds__(256) swa_fwd_kernel(ktx_swa_config c, int T, i
         const float* kj = kt + (size_t)j * DP;
         float s = 0.f;
         for (int d = 0; d < D; d++) s += qh[d] * kj[d];
+        if (dist_bias) s += dist_bias[(size_t)min(p - jpos[j], c.bias_span) * c.heads + h0 + h];
         sc[(size_t)h * KTN + j] = s;      // (scale is folded into q)
       }
     }
@@ -434,8 +519,9 @@ __global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, 
                                                        const bf16_t* __restrict__ kcache, const bf16_t* __restrict__ vcache,
                                                        const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
                                                        const int32_t* __restrict__ page_indptr, const int32_t* __restrict__ page_indices,
-                                                       const float* __restrict__ sink, const float* __restrict__ vcs, int nsplit,
-                                                       float* __restrict__ scratch, OT* __restrict__ out) {
+                                                       const float* __restrict__ sink, const float* __restrict__ dist_bias,
+                                                       const float* __restrict__ vcs, int nsplit, float* __restrict__ scratch,
+                                                       OT* __restrict__ out) {
   constexpr int V = NT * 16;
   extern __shared__ __attribute__((aligned(16))) unsigned char sm_raw[];
   const int H = c.heads, G = c.kv_heads, HPG = H / G, D = c.dim, DPP = D + 8, KS = D / 32;
@@ -450,8 +536,10 @@ __global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, 
   const int p0 = pos0[b];
   const int tok_lo = r0 / HPG, tok_hi = (min(rows_total, r0 + 64) - 1) / HPG;
   const int klo = c.window > 0 ? max(0, p0 + tok_lo - c.window + 1) : 0, khi = p0 + tok_hi + 1;
-  const int per = (((khi - klo + nsplit - 1) / nsplit) + SM_KT - 1) / SM_KT * SM_KT;
-  const int j0 = klo + z * per, j1 = min(khi, j0 + per);
+  // the keys any of the rows sees, as one list: the kept first positions in front of the rows' windows, then the union of the windows
+  const int nfront = min(c.keep_first, klo), nvis = nfront + (khi - klo);
+  const int per = (((nvis + nsplit - 1) / nsplit) + SM_KT - 1) / SM_KT * SM_KT;
+  const int j0 = z * per, j1 = min(nvis, j0 + per);
   const int rw0 = r0 + wave * 16;
   const bool active = rw0 < rows_total;
   // query fragments: lane = (row l16, 8 consecutive entries lq * 8 ..) of every 32-entry step
@@ -478,12 +566,14 @@ __global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, 
   // the four rows this lane holds of the score / output tiles (C layout: row lq * 4 + r, column l16)
   int prow[4], lorow[4];
   bool vrow[4];
+  const float* brow[4];                    // the distance-bias column of the row's head
 #pragma unroll
   for (int r = 0; r < 4; r++) {
     const int cr = rw0 + lq * 4 + r;
     vrow[r] = cr < rows_total;
     prow[r] = p0 + cr / HPG;
     lorow[r] = c.window > 0 ? max(0, prow[r] - c.window + 1) : 0;
+    brow[r] = dist_bias ? dist_bias + g * HPG + cr % HPG : nullptr;
   }
   float mrun[4], lrun[4];
   v4f acc[NT];
@@ -501,7 +591,7 @@ __global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, 
     const int nk = min(SM_KT, j1 - jt);
     __syncthreads();
     if (tid < SM_KT) {
-      const int j = jt + tid;
+      const int u = jt + tid, j = u < nfront ? u : klo + (u - nfront);
       rowidx[tid] = tid < nk ? pages[j / c.page_size] * c.page_size + j % c.page_size : -1;
     }
     __syncthreads();
@@ -533,12 +623,15 @@ __global__ void __launch_bounds__(256) swa_mfma_kernel(ktx_swa_config c, int T, 
           s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qf[kk], b1, s1, 0, 0, 0);
         }
       }
-      const int ja = jt + l16, jb = ja + 16;
+      const int ua = jt + l16, ub = ua + 16;
+      const int ja = ua < nfront ? ua : klo + (ua - nfront), jb = ub < nfront ? ub : klo + (ub - nfront);
 #pragma unroll
       for (int r = 0; r < 4; r++) {
-        const bool oka = vrow[r] && ja < j1 && ja >= lorow[r] && ja <= prow[r];
-        const bool okb = vrow[r] && jb < j1 && jb >= lorow[r] && jb <= prow[r];
-        const float sa = oka ? s0[r] : -INFINITY, sb = okb ? s1[r] : -INFINITY;      // (scale is folded into q)
+        const bool oka = vrow[r] && ua < j1 && (ja >= lorow[r] || ja < c.keep_first) && ja <= prow[r];
+        const bool okb = vrow[r] && ub < j1 && (jb >= lorow[r] || jb < c.keep_first) && jb <= prow[r];
+        float sa = -INFINITY, sb = -INFINITY;      // (scale is folded into q)
+        if (oka) sa = s0[r] + (brow[r] ? brow[r][(size_t)min(prow[r] - ja, c.bias_span) * H] : 0.f);
+        if (okb) sb = s1[r] + (brow[r] ? brow[r][(size_t)min(prow[r] - jb, c.bias_span) * H] : 0.f);
         const float mt = row16_max(fmaxf(sa, sb));
         const float mn = fmaxf(mrun[r], mt);
         const float mb = mn == -INFINITY ? 0.f : mn;
@@ -940,6 +1033,7 @@ static int swa_check(const ktx_swa_config* c, const char* who) {
               std::string(who) + ": heads a multiple of kv_heads, positive sizes, a known cache type");
   KTX_REQUIRE(c->rot_dims >= 0 && c->rot_dims % 2 == 0 && c->rot_dims <= c->dim, std::string(who) + ": rot_dims even and at most dim");
   KTX_REQUIRE(!c->rot_values || c->vdim % 2 == 0, std::string(who) + ": rotated values need an even vdim");
+  KTX_REQUIRE(c->keep_first >= 0 && c->bias_span >= 0, std::string(who) + ": keep_first and bias_span are not negative");
   return 0;
 }
 
@@ -967,6 +1061,40 @@ int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t 
   return 0;
 }
 
+int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
+                      const float* d_conv_w, const float* d_q_norm_w, const float* d_k_norm_w, const int32_t* d_q_indptr,
+                      const int32_t* d_pos0, const int32_t* d_slot, const int32_t* d_tok_req, float* d_conv_state,
+                      const int32_t* d_cache_loc, void* d_kcache, void* d_vcache, float* d_q_out, ktx_stream_t stream) {
+  if (swa_check(cfg, "ktx_swa_conv_prep")) return -1;
+  KTX_REQUIRE(B >= 0 && T >= 0 && d_proj && d_q_indptr && d_pos0 && d_slot && d_tok_req && d_cache_loc && d_kcache && d_vcache && d_q_out,
+              "ktx_swa_conv_prep: null pointer");
+  KTX_REQUIRE(taps >= 0 && taps <= CP_MAX_TAPS && (taps <= 1 || (d_conv_w && d_conv_state)),
+              "ktx_swa_conv_prep: at most 16 taps; a convolution needs its weights and state slots");
+  KTX_REQUIRE(cfg->rot_dims == 0 && !cfg->rot_values, "ktx_swa_conv_prep: no rotation in this form");
+  const int C = cfg->heads * cfg->dim + cfg->kv_heads * (cfg->dim + cfg->vdim);
+  KTX_REQUIRE(ldp >= C, "ktx_swa_conv_prep: rows of q | k | v");
+  KTX_REQUIRE((size_t)C * 4 <= 150 * 1024, "ktx_swa_conv_prep: a token's q | k | v row must fit the LDS");
+  if (T == 0 || B == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)C * 4;
+  if (cfg->cache_dtype == KTX_SEQ_F32) {
+    KTX_HIP(ktx_set_max_lds((const void*)swa_conv_prep_kernel<float>, 150 * 1024));
+    swa_conv_prep_kernel<float><<<T, 256, lds, st>>>(*cfg, taps, d_proj, ldp, d_bias, d_conv_w, d_q_norm_w, d_k_norm_w, d_q_indptr, d_pos0,
+                                                     d_slot, d_tok_req, d_conv_state, d_cache_loc, (float*)d_kcache, (float*)d_vcache, d_q_out);
+  } else {
+    KTX_HIP(ktx_set_max_lds((const void*)swa_conv_prep_kernel<bf16_t>, 150 * 1024));
+    swa_conv_prep_kernel<bf16_t><<<T, 256, lds, st>>>(*cfg, taps, d_proj, ldp, d_bias, d_conv_w, d_q_norm_w, d_k_norm_w, d_q_indptr, d_pos0,
+                                                      d_slot, d_tok_req, d_conv_state, d_cache_loc, (bf16_t*)d_kcache, (bf16_t*)d_vcache,
+                                                      d_q_out);
+  }
+  KTX_HIP(hipGetLastError());
+  if (taps > 1) {      // second launch: the state moves on only after every token of the step has read it
+    conv_state_update_kernel<<<dim3((C + 255) / 256, B), 256, 0, st>>>(C, taps, d_q_indptr, d_pos0, d_slot, d_proj, ldp, d_bias, d_conv_state);
+    KTX_HIP(hipGetLastError());
+  }
+  return 0;
+}
+
 static int swa_merge(const ktx_swa_config* cfg, int T, int nsplit, const float* d_scratch, const float* d_sink, const float* d_vcs,
                      void* d_out, int out_dtype, hipStream_t st) {
   const dim3 mg(T, cfg->heads);
@@ -982,7 +1110,8 @@ static int swa_merge(const ktx_swa_config* cfg, int T, int nsplit, const float* 
 
 int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const void* d_kcache, const void* d_vcache,
                     const int32_t* d_tok_req, const int32_t* d_pos, const int32_t* d_page_indptr, const int32_t* d_page_indices,
-                    const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+                    const float* d_sink, const float* d_dist_bias, const float* d_vcs, int nsplit, float* d_scratch, void* d_out,
+                    int out_dtype, ktx_stream_t stream) {
   if (swa_check(cfg, "ktx_swa_forward")) return -1;
   KTX_REQUIRE(T >= 0 && d_q && d_kcache && d_vcache && d_tok_req && d_pos && d_page_indptr && d_page_indices && d_out && dtype_ok(out_dtype),
               "ktx_swa_forward: null pointer");
@@ -995,7 +1124,7 @@ int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const vo
   int HG = std::min(HPG, std::max(1, 256 * SW_NACC / V));
   int KTN = 64;
   auto lds_of = [&](int hg, int ktn) {
-    return ((size_t)hg * D + (size_t)ktn * (D + 1) + (size_t)ktn * (V + 1) + (size_t)hg * ktn + 3 * (size_t)hg + ktn) * 4;
+    return ((size_t)hg * D + (size_t)ktn * (D + 1) + (size_t)ktn * (V + 1) + (size_t)hg * ktn + 3 * (size_t)hg + 2 * (size_t)ktn) * 4;
   };
   while (KTN > 8 && lds_of(1, KTN) > budget) KTN /= 2;
   while (HG > 1 && lds_of(HG, KTN) > budget) HG = (HG + 1) / 2;
@@ -1008,7 +1137,7 @@ int ktx_swa_forward(const ktx_swa_config* cfg, int T, const float* d_q, const vo
   do {                                                                                                                             \
     KTX_HIP(ktx_set_max_lds((const void*)swa_fwd_kernel<KT, OT>, 150 * 1024));                                                     \
     swa_fwd_kernel<KT, OT><<<grid, 256, lds, st>>>(*cfg, T, HG, parts, KTN, d_q, (const KT*)d_kcache, (const KT*)d_vcache, d_tok_req, \
-                                                   d_pos, d_page_indptr, d_page_indices, d_sink, d_vcs, nsplit, d_scratch, (OT*)d_out); \
+                                                   d_pos, d_page_indptr, d_page_indices, d_sink, d_dist_bias, d_vcs, nsplit, d_scratch, (OT*)d_out); \
   } while (0)
   if (cfg->cache_dtype == KTX_SEQ_F32) {
     if (out_dtype == KTX_SEQ_F32) KTX_SW_GO(float, float);
@@ -1027,15 +1156,16 @@ int ktx_swa_mfma_eligible(const ktx_swa_config* c) {
   if (!c || c->cache_dtype != KTX_SEQ_BF16) return 0;
   if (c->dim % 32 != 0 || c->dim > 32 * SM_KSMAX) return 0;
   const int V = c->vdim;
-  if (!(V == 32 || V == 64 || V == 96 || V == 128 || V == 256)) return 0;
+  if (!((V % 16 == 0 && V >= 16 && V <= 128) || V == 256)) return 0;
   return swa_mfma_lds(*c) <= 150 * 1024;
 }
 
 int ktx_swa_mfma(const ktx_swa_config* cfg, int B, int T, int max_q_len, const float* d_q, const void* d_kcache, const void* d_vcache,
                  const int32_t* d_q_indptr, const int32_t* d_pos0, const int32_t* d_page_indptr, const int32_t* d_page_indices,
-                 const float* d_sink, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype, ktx_stream_t stream) {
+                 const float* d_sink, const float* d_dist_bias, const float* d_vcs, int nsplit, float* d_scratch, void* d_out, int out_dtype,
+                 ktx_stream_t stream) {
   if (swa_check(cfg, "ktx_swa_mfma")) return -1;
-  KTX_REQUIRE(ktx_swa_mfma_eligible(cfg), "ktx_swa_mfma: bf16 caches, dim a multiple of 32 up to 256, vdim 32 / 64 / 96 / 128 / 256");
+  KTX_REQUIRE(ktx_swa_mfma_eligible(cfg), "ktx_swa_mfma: bf16 caches, dim a multiple of 32 up to 256, vdim a multiple of 16 up to 128, or 256");
   KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_q && d_kcache && d_vcache && d_q_indptr && d_pos0 && d_page_indptr &&
                   d_page_indices && d_out && dtype_ok(out_dtype),
               "ktx_swa_mfma: null pointer");
@@ -1054,14 +1184,18 @@ int ktx_swa_mfma(const ktx_swa_config* cfg, int B, int T, int max_q_len, const f
   do {                                                                                                                                \
     KTX_HIP(ktx_set_max_lds((const void*)swa_mfma_kernel<NT, OT>, 150 * 1024));                                                       \
     swa_mfma_kernel<NT, OT><<<grid, 256, lds, st>>>(*cfg, T, row_tiles, d_q, (const bf16_t*)d_kcache, (const bf16_t*)d_vcache,        \
-                                                    d_q_indptr, d_pos0, d_page_indptr, d_page_indices, d_sink, d_vcs, nsplit, d_scratch, \
+                                                    d_q_indptr, d_pos0, d_page_indptr, d_page_indices, d_sink, d_dist_bias, d_vcs, nsplit, d_scratch, \
                                                     (OT*)d_out);                                                                      \
   } while (0)
 #define KTX_SM_NT(OT)                  \
   do {                                 \
-    if (V == 32) KTX_SM_GO(2, OT);     \
+    if (V == 16) KTX_SM_GO(1, OT);     \
+    else if (V == 32) KTX_SM_GO(2, OT); \
+    else if (V == 48) KTX_SM_GO(3, OT); \
     else if (V == 64) KTX_SM_GO(4, OT); \
+    else if (V == 80) KTX_SM_GO(5, OT); \
     else if (V == 96) KTX_SM_GO(6, OT); \
+    else if (V == 112) KTX_SM_GO(7, OT); \
     else if (V == 128) KTX_SM_GO(8, OT); \
     else KTX_SM_GO(16, OT);            \
   } while (0)

@@ -78,6 +78,17 @@ def _sadosun_cache(config, max_tokens, max_requests, dtype, device):
     return KHybridCache(sadosun_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
 
 
+def _vigodra_config(d, dtype):
+    from ktransformers_amd.models.modeling_vigodra import make_vigodra_config
+    return make_vigodra_config(d, dtype)
+
+
+def _vigodra_cache(config, max_tokens, max_requests, dtype, device):
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    from ktransformers_amd.models.modeling_vigodra import vigodra_layer_specs
+    return KHybridCache(vigodra_layer_specs(config), max_tokens, max_requests=max_requests, dtype=dtype, device=device)
+
+
 def _cls(module: str, name: str):
     def get():
         import importlib
@@ -98,6 +109,8 @@ MODEL_REGISTRY = {
                           _pilavik_cache, dtypes=(torch.bfloat16, torch.float32)),
     "Sadosun": ModelEntry(_sadosun_config, _cls("ktransformers_amd.models.modeling_sadosun", "SadosunForCausalLM"), "Sadosun.yaml",
                           _sadosun_cache, dtypes=(torch.bfloat16, torch.float32)),
+    "Vigodra": ModelEntry(_vigodra_config, _cls("ktransformers_amd.models.modeling_vigodra", "VigodraForCausalLM"), "Vigodra.yaml",
+                          _vigodra_cache, dtypes=(torch.bfloat16, torch.float32)),
 }
 
 

@@ -80,9 +80,9 @@ class KScaledEmbedding(BaseInjectedModule):
         t = self.gguf_loader.load_tensor(self.key, device=torch.device(self.device)).to(torch.float32)
         self.w["table"] = (t * self.scale).contiguous()
 
-    def forward(self, tokens: torch.Tensor, positions: torch.Tensor | None = None) -> torch.Tensor:
+    def forward(self, tokens: torch.Tensor, positions: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
         from ktransformers_amd._native_seq import embed_rows
-        return embed_rows(tokens.reshape(-1).to(torch.int32), self.w["table"])
+        return embed_rows(tokens.reshape(-1).to(torch.int32), self.w["table"], out=out)
 
 
 class KTokenSideTable(BaseInjectedModule):

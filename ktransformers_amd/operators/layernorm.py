@@ -95,12 +95,41 @@ class KLayerNormBias(BaseInjectedModule):
         from ktransformers_amd._native_hyb import layer_norm
         return layer_norm(x, self.weight_f32, self.bias_f32, self.eps, rows=rows, out_dtype=out_dtype or self.compute_dtype or torch.float32)
 
+    def post_mix(self, x_in, x_out, y=None, ybias=None, alpha: float = 1.0, stack=None, level: int = 0, depth=None, lp_dtype=None):
+        """BEHIND a sublayer of a post-normed decoder whose residual is scaled: x_out = norm(alpha * x_in + y + ybias), one launch
+        (`ktx_postnorm_mix`).  With `stack` (fp32 [levels, T, W]: the embedding output and every layer's result so far) the normed rows
+        become level `level`, and with `depth` (a KDepthAverage) x_out is the weighted sum of levels 0 .. level instead — what a
+        depth-weighted average hands to the next layer.  Returns what the following products read: x_out itself, or its copy in lp_dtype."""
+        from ktransformers_amd._native_hyb import postnorm_mix
+        return postnorm_mix(x_in, x_out, self.weight_f32, self.bias_f32, self.eps, alpha=alpha, y=y, ybias=ybias, stack=stack, level=level,
+                            dwa=None if depth is None else depth.weights(level + 1), lp_dtype=lp_dtype)
+
     def gated_add(self, x, y=None, ybias=None, gate_logits=None, gate_bias=None, expert_rows=None, pair_pos=None, topk_w=None, next_norm=None):
         import torch
         from ktransformers_amd._native_hyb import gated_norm_add
         nn_ = None if next_norm is None else (next_norm.weight_f32, next_norm.bias_f32, next_norm.eps, next_norm.compute_dtype or torch.float32)
         return gated_norm_add(x, self.weight_f32, self.bias_f32, self.eps, y=y, ybias=ybias, gate_logits=gate_logits, gate_bias=gate_bias,
                               expert_rows=expert_rows, pair_pos=pair_pos, topk_w=topk_w, next_norm=nn_)
+
+
+class KDepthAverage(BaseInjectedModule):
+    """The weights of a depth-weighted average: behind layer i the residual handed on is sum_{j <= i + 1} w[j] X_j over the embedding
+    output X_0 and the layers' results X_1 .. X_(i+1).  The sum itself runs in the launch of the layer's last norm
+    (KLayerNormBias.post_mix).  Checkpoint tensor: the module's key, fp32 [i + 2]."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        object.__setattr__(self, "w_f32", None)
+
+    def load(self):
+        import torch
+        w = self.gguf_loader.load_tensor(self.key, device=torch.device(self.device)).to(torch.float32).reshape(-1).contiguous()
+        object.__setattr__(self, "w_f32", w)
+
+    def weights(self, n: int):
+        if self.w_f32.numel() != n:
+            raise ValueError(f"{self.key}: an average over {n} levels takes {n} weights, the checkpoint has {self.w_f32.numel()}")
+        return self.w_f32
 
 
 class KScalarRMSNorm(BaseInjectedModule):

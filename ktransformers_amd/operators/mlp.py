@@ -169,3 +169,33 @@ class KPolyNormMLP(BaseInjectedModule):
         proj = dense_gemm(h, self._merged[k])
         a = poly_norm(proj[:, :F], self.w["up.b"], self.w["act"], self.eps, out_dtype=self.compute_dtype)
         return dense_gemm(a, self.w["down"]), (proj[:, F:] if rider is not None else None)
+
+
+class KClampedGLUMLP(BaseInjectedModule):
+    """Three-matrix gated feed-forward on an fp32 residual stream whose halves are bounded before they meet:
+    W_down (g sigmoid(slope g) (u + up_shift)), g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit).  gate and up are one product
+    ([gate ; up] merged at load), the activation one launch (include/ktx_hyb.h `ktx_glu_clamp_rows`), fp32 out.  limit (None: unbounded),
+    slope and up_shift are read from the replaced module.  Checkpoint tensors: `<key>.gate`, `<key>.up` [ff, width], `<key>.down`
+    [width, ff]."""
+
+    def __init__(self, key: str, gguf_loader, config, orig_module, prefill_device: str = "cuda", generate_device: str = "cuda", **kwargs):
+        BaseInjectedModule.__init__(self, key, gguf_loader, config, orig_module, prefill_device, generate_device, **kwargs)
+        for name in ("width", "ff", "limit", "slope", "up_shift"):
+            object.__setattr__(self, name, getattr(orig_module, name))
+        object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
+        object.__setattr__(self, "w", {})
+
+    def load(self):
+        dev, cd = torch.device(self.device), self.compute_dtype
+        get = lambda n: self.gguf_loader.load_tensor(f"{self.key}.{n}", device=dev).to(cd)
+        gate, up, down = get("gate"), get("up"), get("down")
+        if tuple(gate.shape) != (self.ff, self.width) or tuple(up.shape) != (self.ff, self.width) or tuple(down.shape) != (self.width, self.ff):
+            raise ValueError(f"{self.key}: tensor shapes do not fit ff={self.ff} width={self.width}")
+        self.w.update(gate_up=torch.cat([gate, up]).contiguous(), down=down.contiguous())
+
+    def forward(self, h: torch.Tensor) -> torch.Tensor:
+        """h [T, width] in the compute type -> fp32 [T, width]."""
+        from ktransformers_amd._native_hyb import glu_clamp_rows
+        from ktransformers_amd._native_seq import dense_gemm
+        a = glu_clamp_rows(dense_gemm(h, self.w["gate_up"]), self.limit, self.slope, self.up_shift, out_dtype=self.compute_dtype)
+        return dense_gemm(a, self.w["down"])

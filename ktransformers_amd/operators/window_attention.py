@@ -13,7 +13,19 @@ operators (operators/attention.py, latent_window_attention.py) for decoders on a
 Rotated, normed keys and rotated values are appended to the KHybridCache's paged key / value caches (spec "kv") by the prep launch;
 prompts, portions and decode steps are one pass over them (include/ktx_swa.h `ktx_swa_prep`, `ktx_swa_mfma` on the matrix cores for
 bf16 caches, `ktx_swa_forward` on the vector ALUs for fp32 and odd sizes).  Angles, scores and softmax are fp32.  window, scale, the
-rotation's base and span, the sink's score, eps and the q / k norm are constructor arguments (read from the replaced module)."""
+rotation's base and span, the sink's score, eps and the q / k norm are constructor arguments (read from the replaced module).
+
+Further options, each off unless the replaced module names it:
+    qkv_bias / out_bias   the projections have biases (`<key>.q.b` ..; the output's is handed to the caller as `out_bias`: it joins the
+                          residual in the norm's launch);
+    conv_taps             a causal convolution over time on every channel of q, k and v directly behind the projections
+                          (`<key>.q.conv` .. [channels, taps]); the last taps - 1 projected rows of a sequence are state (spec "conv");
+    proj_norm             q and k are RMS-normed over their WHOLE projection (all heads at once) with weights `<key>.q.norm`, `<key>.k.norm`;
+    dist_far              a learned bias by distance is added to the scaled score, `<key>.rel` [rows, heads]: distances below rows / 2
+                          have a row each, the rest share rows on a logarithmic scale that reaches the last row at distance dist_far;
+    keep_first            the sequence's first positions stay visible behind the window;
+    sink = "learned"      the sink's score is `<key>.sink` [heads].
+With any of the first three the prep is `ktx_swa_conv_prep` (no rotation in that form)."""
 from __future__ import annotations
 
 import torch
@@ -34,12 +46,36 @@ class KWindowGQAttention(BaseInjectedModule):
         for name in ("heads", "kv_heads", "dim", "vdim", "rot_dims", "rot_base", "rot_values", "qk_norm", "sink_score", "scale", "window",
                      "eps", "width"):
             object.__setattr__(self, name, getattr(o, name))
+        for name, default in (("qkv_bias", False), ("out_bias_on", False), ("conv_taps", 0), ("proj_norm", False), ("dist_far", None),
+                              ("keep_first", 0), ("sink", None)):
+            object.__setattr__(self, name, getattr(o, name, default))
+        object.__setattr__(self, "conv_form", bool(self.qkv_bias or self.conv_taps or self.proj_norm))
+        if self.conv_form and (self.rot_dims or self.rot_values or self.qk_norm):
+            raise ValueError(f"{key}: biases, a convolution or whole-projection norms go with un-rotated, un-normed heads")
         object.__setattr__(self, "compute_dtype", getattr(config, "compute_dtype", torch.bfloat16))
         object.__setattr__(self, "w", {})
         object.__setattr__(self, "_cfg", {})
 
     def state_spec(self) -> dict:
-        return {"kv": (self.kv_heads, self.dim, self.vdim)}
+        spec = {"kv": (self.kv_heads, self.dim, self.vdim)}
+        if self.conv_taps > 1:
+            spec["conv"] = (self.heads * self.dim + self.kv_heads * (self.dim + self.vdim), self.conv_taps)
+        return spec
+
+    @property
+    def out_bias(self):
+        return self.w.get("o_b")
+
+    @staticmethod
+    def distance_rows(rows: int, far: float) -> list:
+        """Row of a [rows, heads] distance table for each distance 0 .. ceil(far): the first rows / 2 distances have a row each, the rest
+        share rows on a logarithmic scale that reaches the last row at distance `far` (every larger distance reads the last row)."""
+        import math
+        half = rows // 2
+        out = []
+        for n in range(int(math.ceil(far)) + 1):
+            out.append(n if n < half else min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(far / half) * (rows - half)))))
+        return out
 
     def load(self):
         ld, dev, cd = self.gguf_loader, torch.device(self.device), self.compute_dtype
@@ -55,31 +91,60 @@ class KWindowGQAttention(BaseInjectedModule):
         self.w["inv_freq"] = f64(self.rot_dims) if self.rot_dims else None
         self.w["v_inv_freq"] = f64(V) if self.rot_values else None
         self.w["sink"] = None if self.sink_score is None else torch.full((H,), float(self.sink_score), dtype=torch.float32, device=dev)
+        f32 = lambda n: ld.load_tensor(f"{self.key}.{n}", device=dev).to(torch.float32).contiguous()
+        if self.sink == "learned":
+            self.w["sink"] = f32("sink").reshape(-1)
+            if self.w["sink"].numel() != H:
+                raise ValueError(f"{self.key}.sink: one score per head")
+        if self.qkv_bias:
+            self.w["qkv_b"] = torch.cat([f32("q.b"), f32("k.b"), f32("v.b")]).contiguous()
+        if self.out_bias_on:
+            self.w["o_b"] = f32("o.b")
+        if self.conv_taps:
+            self.w["conv"] = torch.cat([f32("q.conv"), f32("k.conv"), f32("v.conv")]).contiguous()
+            if tuple(self.w["conv"].shape) != ((H + G) * D + G * V, self.conv_taps):
+                raise ValueError(f"{self.key}: convolution weights must be [channels, {self.conv_taps}]")
+        if self.proj_norm:
+            self.w["q_norm"], self.w["k_norm"] = f32("q.norm").reshape(-1), f32("k.norm").reshape(-1)
+        self.w["dist_bias"] = None
+        if self.dist_far is not None:
+            rel, far = f32("rel"), float(self.dist_far)
+            rows = rel.shape[0]
+            if rel.dim() != 2 or rel.shape[1] != H or rows < 2 or far <= rows // 2:
+                raise ValueError(f"{self.key}.rel: expected [rows >= 2, {H}] and a far distance beyond rows / 2")
+            # the table by DISTANCE: the kernels index it with min(i - j, its last row)
+            self.w["dist_bias"] = rel[torch.tensor(self.distance_rows(rows, far), device=dev)].contiguous()
 
     def _config(self, cache):
         from ktransformers_amd._native_swa import swa_config
         k = (cache.page_size, cache.dtype)
         if k not in self._cfg:
             self._cfg[k] = swa_config(self.heads, self.kv_heads, self.dim, self.vdim, self.rot_dims, self.rot_values, self.qk_norm,
-                                      self.eps, self.scale, self.window or 0, cache.page_size, cache.dtype)
+                                      self.eps, self.scale, self.window or 0, cache.page_size, cache.dtype, keep_first=self.keep_first,
+                                      bias_span=0 if self.w["dist_bias"] is None else self.w["dist_bias"].shape[0] - 1)
         return self._cfg[k]
 
     def forward(self, h: torch.Tensor, batch, cache, cache_idx: int) -> torch.Tensor:
         """h [T, width] in the compute type -> W_o(attention) fp32 [T, width]; the step's key and value rows are appended to the cache."""
         from ktransformers_amd._native_seq import dense_gemm
-        from ktransformers_amd._native_swa import swa_forward, swa_mfma, swa_mfma_eligible, swa_prep
+        from ktransformers_amd._native_swa import swa_conv_prep, swa_forward, swa_mfma, swa_mfma_eligible, swa_prep
         H, G, D = self.heads, self.kv_heads, self.dim
         cfg, T = self._config(cache), h.shape[0]
         kc, vc = cache.k_caches[cache_idx], cache.v_caches[cache_idx]
         proj = dense_gemm(h, self.w["qkv"])
-        q, vcs = swa_prep(cfg, proj, 0, H * D, (H + G) * D, self.w["inv_freq"], self.w["v_inv_freq"], batch.positions, batch.cache_loc, kc, vc)
-        span = batch.max_kv_len if not self.window else min(batch.max_kv_len, self.window + batch.max_q_len)
+        if self.conv_form:
+            q, vcs = swa_conv_prep(cfg, proj, self.w.get("qkv_b"), self.w.get("conv"), self.w.get("q_norm"), self.w.get("k_norm"), batch,
+                                   cache.conv[cache_idx] if self.conv_taps > 1 else None, kc, vc), None
+        else:
+            q, vcs = swa_prep(cfg, proj, 0, H * D, (H + G) * D, self.w["inv_freq"], self.w["v_inv_freq"], batch.positions, batch.cache_loc, kc, vc)
+        bias = self.w["dist_bias"]
+        span = batch.max_kv_len if not self.window else min(batch.max_kv_len, self.window + self.keep_first + batch.max_q_len)
         if self.USE_MATRIX_CORES and kc.dtype == torch.bfloat16 and swa_mfma_eligible(cfg):
             blocks = batch.B * G * ((batch.max_q_len * (H // G) + 63) // 64)
             nsplit = max(1, min(self.TARGET_WORKGROUPS // max(blocks, 1), (span + self.KEYS_PER_SPLIT - 1) // self.KEYS_PER_SPLIT))
-            o = swa_mfma(cfg, q, kc, vc, batch, self.w["sink"], vcs, nsplit=nsplit, out_dtype=self.compute_dtype)
+            o = swa_mfma(cfg, q, kc, vc, batch, self.w["sink"], vcs, nsplit=nsplit, out_dtype=self.compute_dtype, dist_bias=bias)
         else:
-            span = batch.max_kv_len if not self.window else min(batch.max_kv_len, self.window)
+            span = batch.max_kv_len if not self.window else min(batch.max_kv_len, self.window + self.keep_first)
             nsplit = max(1, min(self.TARGET_WORKGROUPS // max(T * G, 1), (span + self.KEYS_PER_SPLIT - 1) // self.KEYS_PER_SPLIT))
-            o = swa_forward(cfg, q, kc, vc, batch, self.w["sink"], vcs, nsplit=nsplit, out_dtype=self.compute_dtype)
+            o = swa_forward(cfg, q, kc, vc, batch, self.w["sink"], vcs, nsplit=nsplit, out_dtype=self.compute_dtype, dist_bias=bias)
         return dense_gemm(o, self.w["o"])
