@@ -59,6 +59,26 @@ def distance_bias_matrix(T: int, column, far: float):
     return by_dist[(i - j).clamp(min=0)] * (j <= i)
 
 
+def attention_core(q, k, v, scale, size=None, keep_first=0, rel=None, far=None, sink=None):
+    """q [T, H, D], k [T, G, D], v [T, G, V] of ONE sequence -> [T, H, V]: softmax over the visible keys of scale q.k + rel[bucket(i - j), head]
+    and, with sink [H], one extra score per head that only enlarges the denominator."""
+    T, H, _ = q.shape
+    G = k.shape[1]
+    see = visible_matrix(T, size, keep_first)
+    out = torch.zeros(T, H, v.shape[2], dtype=q.dtype)
+    for hd in range(H):
+        g = hd // (H // G)
+        s = (q[:, hd] @ k[:, g].T) * scale                            # [i, j]
+        if rel is not None:
+            s = s + distance_bias_matrix(T, rel[:, hd], far)
+        s = s.masked_fill(~see, float("-inf"))
+        if sink is not None:                                          # one more column whose weight is dropped
+            s = torch.cat([s, sink[hd].expand(T, 1)], dim=1)
+        w = torch.softmax(s, dim=1)[:, :T]
+        out[:, hd] = w @ v[:, g]
+    return out
+
+
 def biased_window_attention(P, pre, c, h, eps):
     """Grouped-query attention without rotation: q, k, v = biased projections, each followed by a causal convolution over time;
     q and k are RMS-normed over their WHOLE projection (all heads at once) with a weight; score = scale q.k + table[bucket(i - j), head];
@@ -75,20 +95,7 @@ def biased_window_attention(P, pre, c, h, eps):
     q = rms_norm(q, P[pre + "q.norm"], eps).view(T, H, D)
     k = rms_norm(k, P[pre + "k.norm"], eps).view(T, G, D)
     v = v.view(T, G, V)
-    rel = P.get(pre + "rel")
-    sink = P.get(pre + "sink")
-    see = visible_matrix(T, size, keep)
-    out = torch.zeros(T, H, V, dtype=h.dtype)
-    for hd in range(H):
-        g = hd // (H // G)
-        s = (q[:, hd] @ k[:, g].T) * c["scale"]                       # [i, j]
-        if rel is not None:
-            s = s + distance_bias_matrix(T, rel[:, hd], c["bias_max"])
-        s = s.masked_fill(~see, float("-inf"))
-        if sink is not None:                                          # one more column whose weight is dropped
-            s = torch.cat([s, sink[hd].expand(T, 1)], dim=1)
-        w = torch.softmax(s, dim=1)[:, :T]
-        out[:, hd] = w @ v[:, g]
+    out = attention_core(q, k, v, c["scale"], size, keep, P.get(pre + "rel"), c.get("bias_max"), P.get(pre + "sink"))
     return out.reshape(T, H * V) @ P[pre + "o"].T + P[pre + "o.b"]
 
 
@@ -185,3 +192,77 @@ def forward(P, cfg, tokens, dtype=torch.float64, return_layers=False):
         trail.append(x)
     logits = layer_norm(x, P["final.norm"], P["final.norm.b"], eps) @ P["head"].T
     return (logits, torch.stack(trail)) if return_layers else logits
+
+
+# ---- small configurations and random checkpoints for the tests ---------------------------------------------------------------------
+def attention_layer(heads=4, kv_heads=2, dim=16, vdim=16, window=12, keep_first=2, conv=3, bias_max=20, scale=None, mlp="dense"):
+    m = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else dim ** -0.5,
+         "conv": conv, "bias_max": bias_max}
+    if window:
+        m["mask"] = {"size": window, "keep_first": keep_first}
+    return {"type": "attention", "mixer": m, "mlp": dense_mlp() if mlp == "dense" else mlp}
+
+
+def latent_layer(heads=2, dim=8, rot_dim=8, vdim=12, kv_rank=16, window=10, base=10000.0, rot_dims=None, scale=None, kv_from=None, mlp="dense"):
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank,
+         "scale": scale if scale is not None else (dim + rot_dim) ** -0.5, "rot": {"base": base, "dims": rot_dim if rot_dims is None else rot_dims}}
+    if window:
+        m["mask"] = {"size": window}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": "latent_attention", "mixer": m, "mlp": dense_mlp() if mlp == "dense" else mlp}
+
+
+def dense_mlp(ff=40, limit=1.5):
+    return {"kind": "dense", "ff": ff, "limit": limit}
+
+
+def make_config(layers, width=32, vocab=61, eps=1e-5, alpha=1.7, scale=3.0):
+    return {"architecture": "Vigodra", "width": width, "vocab": vocab, "norm": {"eps": eps}, "embedding": {"scale": scale},
+            "postln_alpha": alpha, "layers": layers}
+
+
+def random_checkpoint(cfg: dict, seed: int = 0, rel_rows: int = 8) -> dict:
+    """Random bf16-representable weights with the checkpoint's tensor names for a config of the design."""
+    g = torch.Generator().manual_seed(seed)
+    W = cfg["width"]
+
+    def mat(o, i, s=None):
+        return (torch.randn(o, i, generator=g) * (s if s is not None else 1.0 / math.sqrt(i))).to(torch.bfloat16)
+
+    def vec(n, mean=0.0, s=0.1):
+        return (mean + torch.randn(n, generator=g) * s).to(torch.bfloat16)
+
+    P = {"embed": mat(cfg["vocab"], W, 1.0), "head": mat(cfg["vocab"], W), "final.norm": vec(W, 1.0, 0.2), "final.norm.b": vec(W)}
+    for li, layer in enumerate(cfg["layers"]):
+        p, m = f"l{li}.", layer["mixer"]
+        P[p + "norm1"], P[p + "norm1.b"] = vec(W, 1.0, 0.2), vec(W)
+        if layer["type"] == "attention":
+            H, G, D, V, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], int(m.get("conv") or 0)
+            for n, rows in (("q", H * D), ("k", G * D), ("v", G * V)):
+                P[p + f"mix.{n}"], P[p + f"mix.{n}.b"] = mat(rows, W), vec(rows, 0.0, 0.3)
+                if K:
+                    P[p + f"mix.{n}.conv"] = mat(rows, K, 0.6)
+            P[p + "mix.q.norm"], P[p + "mix.k.norm"] = vec(H * D, 1.0, 0.3), vec(G * D, 1.0, 0.3)
+            if m.get("bias_max") is not None:
+                # (the far distance must lie beyond half the rows)
+                P[p + "mix.rel"] = mat(rel_rows if m["bias_max"] > rel_rows // 2 else 2, H, 1.0)
+            P[p + "mix.sink"] = vec(H, 0.0, 1.0)
+            P[p + "mix.o"], P[p + "mix.o.b"] = mat(W, H * V), vec(W, 0.0, 0.3)
+        else:
+            H, D, R, V, L = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+            P[p + "mix.q"] = mat(H * (D + R), W)
+            if m.get("kv_from") is None:
+                P[p + "mix.dkv"], P[p + "mix.dkv.norm"] = mat(L + R, W), vec(L, 1.0, 0.3)
+            P[p + "mix.uk"], P[p + "mix.uv"] = mat(H * D, L), mat(H * V, L)
+            P[p + "mix.g"], P[p + "mix.o"] = mat(H * V, W), mat(W, H * V)
+        c = layer.get("mlp")
+        if c:
+            P[p + "norm2"], P[p + "norm2.b"] = vec(W, 1.0, 0.2), vec(W)
+            P[p + "mlp.gate"], P[p + "mlp.up"], P[p + "mlp.down"] = mat(c["ff"], W, 2.0 / math.sqrt(W)), mat(c["ff"], W, 2.0 / math.sqrt(W)), mat(W, c["ff"])
+        P[p + "dwa"] = (torch.randn(li + 2, generator=g) * 0.5 + torch.nn.functional.one_hot(torch.tensor(li + 1), li + 2)).to(torch.bfloat16)
+    return P
+
+
+def as_double(P: dict) -> dict:
+    return {k: (v.double() if v.is_floating_point() else v) for k, v in P.items()}

@@ -17,6 +17,7 @@ PAIRS = [("ktx_moe_config", "_MoeConfig", "ktx_moe.h"), ("ktx_linear_config", "_
          ("ktx_sigattn_config", "_SigAttnConfig", "ktx_seq.h"), ("ktx_mlstm_config", "_MlstmConfig", "ktx_seq.h"),
          # (ktransformers_amd/_native_hyb.py, _native_swa.py)
          ("ktx_delta_config", "_DeltaConfig", "ktx_hyb.h"), ("ktx_latattn_config", "_LatAttnConfig", "ktx_hyb.h"),
+         ("ktx_postnorm_args", "_PostNormArgs", "ktx_hyb.h"),
          ("ktx_resid_args", "_ResidArgs", "ktx_swa.h"), ("ktx_swa_config", "_SwaConfig", "ktx_swa.h"),
          ("ktx_ssm_config", "_SsmConfig", "ktx_swa.h")]
 
