@@ -2121,6 +2121,141 @@ def run_sadosun(args, dev):
     print(json.dumps(line), flush=True)
 
 
+# ---------------------------------------------------------------------------------------------------------------------
+# --vigodra: the post-normed family with a depth-weighted average, a biased grouped-query window attention behind convolved projections
+# and a gated latent window attention with shared latent rows (models/modeling_vigodra.py) at a few layer sizes, beside Sadosun — the
+# closest existing family: the same fp32 residual, cache manager, step function and graph replay, and the same grouped-query
+# window-attention kernels with a sink — at equal width and depth
+# ---------------------------------------------------------------------------------------------------------------------
+VIGODRA_SIZES = {
+    # per block of 4 layers: latent attention, attention, attention, latent attention reading the first layer's rows; dense feed-forwards
+    "w1024": dict(width=1024, heads=8, kv_heads=2, dim=128, vdim=128, window=1024, keep_first=4, rel_rows=32, l_heads=8, l_dim=64, l_rot=32,
+                  l_vdim=64, kv_rank=256, ff=2816, sadosun="w1024"),
+    "w2048": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, window=1024, keep_first=4, rel_rows=32, l_heads=16, l_dim=64, l_rot=32,
+                  l_vdim=64, kv_rank=256, ff=5632, sadosun="w2048"),
+    "w4096": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, window=2048, keep_first=4, rel_rows=32, l_heads=32, l_dim=128, l_rot=64,
+                  l_vdim=128, kv_rank=512, ff=11008, sadosun="w4096"),
+}
+
+
+def vigodra_config(sz, n_layers, vocab=32000):
+    attn = {"type": "attention", "mixer": {"heads": sz["heads"], "kv_heads": sz["kv_heads"], "dim": sz["dim"], "vdim": sz["vdim"],
+                                           "scale": sz["dim"] ** -0.5, "conv": 4, "bias_max": sz["window"],
+                                           "mask": {"size": sz["window"], "keep_first": sz["keep_first"]}}}
+    lat = {"heads": sz["l_heads"], "dim": sz["l_dim"], "rot_dim": sz["l_rot"], "vdim": sz["l_vdim"], "kv_rank": sz["kv_rank"],
+           "scale": (sz["l_dim"] + sz["l_rot"]) ** -0.5, "mask": {"size": sz["window"]}, "rot": {"base": 10000.0, "dims": sz["l_rot"]}}
+    mlp = {"kind": "dense", "ff": sz["ff"], "limit": 7.0}
+    layers = []
+    for i in range(n_layers):
+        if i % 4 in (1, 2):
+            layers.append(dict(attn, mlp=mlp))
+        else:
+            layers.append({"type": "latent_attention", "mixer": dict(lat, **({"kv_from": i - 3} if i % 4 == 3 else {})), "mlp": mlp})
+    return {"architecture": "Vigodra", "width": sz["width"], "vocab": vocab, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+            "postln_alpha": 2.0, "layers": layers, "_rel_rows": sz["rel_rows"]}
+
+
+class VigRandomLoader(HybRandomLoader):
+    """Random bf16 weights by tensor name for a Vigodra config (names and shapes of models/modeling_vigodra.py's checkpoint)."""
+
+    def __init__(self, cfg, dev):
+        self.dev, self.tensor_device_map, self.shapes = dev, {}, {}
+        W, S = cfg["width"], self.shapes
+        S.update({"embed": (cfg["vocab"], W), "head": (cfg["vocab"], W), "final.norm": (W,), "final.norm.b": (W,)})
+        for i, L in enumerate(cfg["layers"]):
+            p, m, c = f"l{i}.", L["mixer"], L.get("mlp")
+            for n in ("norm1",) + (("norm2",) if c else ()):
+                S[p + n] = S[p + n + ".b"] = (W,)
+            S[p + "dwa"] = (i + 2,)
+            if L["type"] == "attention":
+                H, G, D, V, K = m["heads"], m["kv_heads"], m["dim"], m["vdim"], m["conv"]
+                for n, rows in (("q", H * D), ("k", G * D), ("v", G * V)):
+                    S.update({p + f"mix.{n}": (rows, W), p + f"mix.{n}.b": (rows,), p + f"mix.{n}.conv": (rows, K)})
+                S.update({p + "mix.q.norm": (H * D,), p + "mix.k.norm": (G * D,), p + "mix.rel": (cfg["_rel_rows"], H), p + "mix.sink": (H,),
+                          p + "mix.o": (W, H * V), p + "mix.o.b": (W,)})
+            else:
+                H, D, R, V, Lr = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+                S.update({p + "mix.q": (H * (D + R), W), p + "mix.uk": (H * D, Lr), p + "mix.uv": (H * V, Lr), p + "mix.g": (H * V, W),
+                          p + "mix.o": (W, H * V)})
+                if m.get("kv_from") is None:
+                    S.update({p + "mix.dkv": (Lr + R, W), p + "mix.dkv.norm": (Lr,)})
+            if c:
+                S.update({p + "mlp.gate": (c["ff"], W), p + "mlp.up": (c["ff"], W), p + "mlp.down": (W, c["ff"])})
+
+    def load_tensor(self, name, device="cpu"):
+        import zlib
+        shape = self.shapes[name]
+        g = torch.Generator(device=self.dev)
+        g.manual_seed(zlib.crc32(name.encode()))
+        t = torch.randn(shape, generator=g, device=self.dev, dtype=torch.bfloat16)
+        leaf = name.rsplit(".", 1)[-1]
+        if leaf in ("norm1", "norm2", "norm"):
+            return t.mul_(0.1).add_(1.0)
+        if leaf == "dwa":
+            return t.mul_(0.1).add_(1.0 / shape[0])
+        if leaf == "conv":
+            return t.mul_(0.5)
+        if leaf in ("rel", "sink"):
+            return t
+        if len(shape) == 1 or name == "embed":
+            return t.mul_(0.1) if name.endswith(".b") else t
+        return t.mul_(shape[-1] ** -0.5)
+
+
+class VigKernelTimer(SwaKernelTimer):
+    """HIP events around every binding a Vigodra step calls."""
+    HYB = ("layer_norm", "postnorm_mix", "glu_clamp_rows", "sigmoid_gate_rows", "latattn_prep", "latattn_forward", "latattn_mfma", "head_gemm")
+    SWA = ("swa_conv_prep", "swa_forward", "swa_mfma")
+
+    def _cost(self, name, a, kw, out):
+        nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0
+        if name == "postnorm_mix":
+            x = a[0]
+            levels = (kw.get("level", 0) + 1) if kw.get("dwa") is not None else (1 if kw.get("stack") is not None else 0)
+            return name, 0.0, (2 + levels) * nb(x) + nb(kw.get("y")) + (nb(out) if out is not a[1] else 0)
+        return super()._cost(name, a, kw, out)
+
+
+def run_vigodra(args, dev):
+    """Prefill (one prompt of --prefill-tokens) and decode (batch 1 and 8 at a 2048-token context) throughput of Vigodra at
+    VIGODRA_SIZES, each beside Sadosun of equal width and depth, with a per-kernel table and the fraction of its roofline (bf16 MFMA
+    peak or HBM peak, whichever bounds).  Random weights, synthetic tokens.  Prints one JSON line; the whole record goes to
+    bench_vigodra.json beside this file."""
+    n_layers, T, ctx = args.layers or 4, args.prefill_tokens, 2048
+    sizes = [s for s in (args.vigodra.split(",") if args.vigodra != "all" else VIGODRA_SIZES) if s in VIGODRA_SIZES]
+    record = {"metric": "vigodra_prefill_decode", "unit": "tok/s", "layers": n_layers, "prefill_tokens": T, "decode_ctx": ctx,
+              "dtype": "bf16 weights / activations / key, value and latent caches, fp32 residual, norms, scores", "data": "synthetic",
+              "sizes": {}}
+    for name in sizes:
+        sz = VIGODRA_SIZES[name]
+        cfg = vigodra_config(sz, n_layers)
+        loader = VigRandomLoader(cfg, dev)
+        res = family_measure(args, dev, cfg, loader, VigKernelTimer, sz["window"] + sz["keep_first"], T, ctx)
+        active = loader.active_params(cfg)
+        res["weights_GB"] = res["active_weights_GB"] = round(active * 2 / 1e9, 3)
+        res["decode_bs1"]["frac_of_hbm_peak"] = round(active * 2 / (res["decode_bs1"]["ms_per_step"] * 1e-3) / (HBM_PEAK_GBS * 1e9), 4)
+        try:
+            ssz = SADOSUN_SIZES[sz["sadosun"]]
+            scfg = sadosun_config(ssz, n_layers)
+            sl = SwaRandomLoader(scfg, dev)
+            res["sadosun"] = family_measure(args, dev, scfg, sl, SwaKernelTimer, ssz["window"], T, ctx)
+            res["sadosun"]["active_weights_GB"] = round((sl.active_params(scfg) - math.prod(sl.shapes.get("side.embed", (0,)))) * 2 / 1e9, 3)
+        except Exception as e:      # the comparison must not lose the new family's numbers
+            res["sadosun"] = {"error": f"{type(e).__name__}: {e}"}
+        record["sizes"][name] = res
+        log(f"[vigodra] {name}: prefill {res['prefill']['tok_s']} tok/s, decode bs1 {res['decode_bs1']['tok_s']} tok/s, "
+            f"bs8 {res['decode_bs8']['tok_s']} tok/s")
+    with open(os.path.join(ROOT, "bench_vigodra.json"), "w") as f:
+        json.dump(record, f, indent=1)
+    line = {"metric": record["metric"], "unit": "tok/s", "layers": n_layers, "data": "synthetic",
+            "sizes": {k: {"prefill": v["prefill"]["tok_s"], "decode_bs1": v["decode_bs1"]["tok_s"], "decode_bs8": v["decode_bs8"]["tok_s"],
+                          "sadosun_prefill": v["sadosun"].get("prefill", {}).get("tok_s"),
+                          "sadosun_decode_bs1": v["sadosun"].get("decode_bs1", {}).get("tok_s"),
+                          "sadosun_decode_bs8": v["sadosun"].get("decode_bs8", {}).get("tok_s")}
+                      for k, v in record["sizes"].items()}}
+    print(json.dumps(line), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -2169,6 +2304,11 @@ def main():
                          "attention with rotated values + selective scan, a softmax-routed mixture with identity experts) at layer sizes "
                          "from SADOSUN_SIZES (comma-separated, or 'all'), beside Pilavik of equal width and depth; one JSON line, detail in "
                          "bench_sadosun.json")
+    ap.add_argument("--vigodra", default="", metavar="SIZES",
+                    help="instead of the default workload: prefill / decode throughput of the Vigodra family (post-normed residual with a "
+                         "depth-weighted average, biased grouped-query window attention behind convolved projections, gated latent window "
+                         "attention with shared latent rows, a bounded GLU) at layer sizes from VIGODRA_SIZES (comma-separated, or 'all'), "
+                         "beside Sadosun of equal width and depth; one JSON line, detail in bench_vigodra.json")
     ap.add_argument("--pmc-child", action="store_true", help=argparse.SUPPRESS)
     ap.add_argument("--trace-child", action="store_true", help=argparse.SUPPRESS)
     args = ap.parse_args()
@@ -2198,6 +2338,10 @@ def main():
     if args.sadosun:
         torch.cuda.set_device(dev)
         run_sadosun(args, dev)
+        return
+    if args.vigodra:
+        torch.cuda.set_device(dev)
+        run_vigodra(args, dev)
         return
     torch.cuda.set_device(dev)
     if args.pmc_child:

@@ -105,8 +105,10 @@ int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t 
  *             zero otherwise; taps <= 1: y = u, times conv_w when given)
  *   q = y_q / sqrt(mean(y_q^2) + eps) * q_norm_w * scale over ALL heads dim entries at once (q_norm_w fp32 [heads dim] or NULL: no norm),
  *   k likewise with k_norm_w over kv_heads dim entries; q -> q_out fp32 [T][heads][dim], k and v = y_v -> cache rows cache_loc[t].
- * Then (second launch) conv_state[slot[b]] = the last taps - 1 inputs u of request b.  cfg: rot_dims = 0, rot_values = 0; taps <= 16. */
-int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
+ * Then (second launch) conv_state[slot[b]] = the last taps - 1 inputs u of request b; with max_q_len == 1 (no request brings more than
+ * one token), 2 .. 4 taps and channel counts that are multiples of 4 the state moves on in the first launch.  cfg: rot_dims = 0,
+ * rot_values = 0; taps <= 16. */
+int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int max_q_len, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
                       const float* d_conv_w, const float* d_q_norm_w, const float* d_k_norm_w, const int32_t* d_q_indptr,
                       const int32_t* d_pos0, const int32_t* d_slot, const int32_t* d_tok_req, float* d_conv_state,
                       const int32_t* d_cache_loc, void* d_kcache, void* d_vcache, float* d_q_out, ktx_stream_t stream);

@@ -36,7 +36,7 @@ lib.ktx_resid_norm.argtypes = [_I, _I, _P, C.POINTER(_ResidArgs), _P]
 lib.ktx_input_conv.argtypes = [_I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _I, _P]
 lib.ktx_rows_mul_lookup.argtypes = [_I, _I, _P, _L, _P, _I, _L, _I, _P, _P, _I, _P]
 lib.ktx_swa_prep.argtypes = [C.POINTER(_SwaConfig), _I, _P, _L, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P]
-lib.ktx_swa_conv_prep.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _P, _L] + [_P] * 14
+lib.ktx_swa_conv_prep.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _I, _P, _L] + [_P] * 14
 lib.ktx_swa_forward.argtypes = [C.POINTER(_SwaConfig), _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
 lib.ktx_swa_mfma_eligible.argtypes = [C.POINTER(_SwaConfig)]
 lib.ktx_swa_mfma.argtypes = [C.POINTER(_SwaConfig), _I, _I, _I, _P, _P, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P, _P, _I, _P]
@@ -199,7 +199,7 @@ def swa_conv_prep(cfg: _SwaConfig, proj: torch.Tensor, bias: torch.Tensor | None
             (taps > 1 and (conv_state is None or tuple(conv_state.shape[1:]) != (taps - 1, Cn))):
         raise KtxError("swa_conv_prep: shapes do not fit")
     q = torch.empty((T, nq), dtype=torch.float32, device=proj.device)
-    check(lib.ktx_swa_conv_prep(C.byref(cfg), batch.B, T, taps, pp, ldp, _ptr(bias), _ptr(conv_w), _ptr(q_norm_w), _ptr(k_norm_w),
+    check(lib.ktx_swa_conv_prep(C.byref(cfg), batch.B, T, int(batch.max_q_len), taps, pp, ldp, _ptr(bias), _ptr(conv_w), _ptr(q_norm_w), _ptr(k_norm_w),
                                 batch.q_indptr.data_ptr(), batch.pos0.data_ptr(), batch.slot.data_ptr(), batch.tok_req.data_ptr(),
                                 _ptr(conv_state), batch.cache_loc.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), q.data_ptr(),
                                 _stream_ptr(proj.device)))

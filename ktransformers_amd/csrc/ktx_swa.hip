@@ -300,6 +300,97 @@ __global__ void __launch_bounds__(256) swa_conv_prep_kernel(ktx_swa_config c, in
   }
 }
 
+// The same prep for 2 .. 4 taps and channel counts that are multiples of 4 (q, k and v each): a thread owns FOUR neighbouring channels
+// (16-byte loads of the projections, the state rows and the taps), requests everything a group needs before it uses any of it, and —
+// in steps where every request brings exactly one token (`one_token`) — moves the slot's state on itself: the token's workgroup is the
+// only reader of its slot, and a thread reads and writes only its own channels.
+template <typename KT, int TAPS>
+__global__ void __launch_bounds__(256) swa_conv_prep_vec_kernel(ktx_swa_config c, const float* __restrict__ proj, int64_t ldp,
+                                                                const float* __restrict__ bias, const float* __restrict__ cw,
+                                                                const float* __restrict__ qw, const float* __restrict__ kw,
+                                                                const int32_t* __restrict__ q_indptr, const int32_t* __restrict__ pos0,
+                                                                const int32_t* __restrict__ slot, const int32_t* __restrict__ tok_req,
+                                                                float* __restrict__ conv_state, int one_token,
+                                                                const int32_t* __restrict__ cache_loc, KT* __restrict__ kcache,
+                                                                KT* __restrict__ vcache, float* __restrict__ q_out) {
+  extern __shared__ __attribute__((aligned(16))) float row[];      // [H * D | G * D | G * V]
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int nq = c.heads * c.dim, nk = c.kv_heads * c.dim, nv = c.kv_heads * c.vdim, C = nq + nk + nv;
+  const int b = tok_req[t], i = t - q_indptr[b];
+  const bool carried = pos0[b] > 0;
+  float* st = conv_state + (size_t)slot[b] * (TAPS - 1) * C;
+  const float4 zero4 = make_float4(0.f, 0.f, 0.f, 0.f);
+  float sq = 0.f, sk = 0.f;
+  for (int e = tid * 4; e < C; e += 1024) {
+    float4 u[TAPS], w[4];
+    const float4 be = bias ? *reinterpret_cast<const float4*>(bias + e) : zero4;
+#pragma unroll
+    for (int j = 0; j < TAPS; j++) {
+      const int ii = i - (TAPS - 1) + j;
+      if (ii >= 0) u[j] = *reinterpret_cast<const float4*>(proj + (size_t)(t - (TAPS - 1) + j) * ldp + e);
+      else if (carried) u[j] = *reinterpret_cast<const float4*>(st + (size_t)(TAPS - 1 + ii) * C + e);
+      else u[j] = zero4;
+    }
+#pragma unroll
+    for (int n = 0; n < 4; n++) {      // the taps of channel e + n: TAPS consecutive floats
+      if constexpr (TAPS == 4) {
+        w[n] = *reinterpret_cast<const float4*>(cw + (size_t)(e + n) * 4);
+      } else {
+        const float* wp = cw + (size_t)(e + n) * TAPS;
+        w[n] = make_float4(wp[0], wp[1], TAPS > 2 ? wp[2] : 0.f, 0.f);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TAPS; j++) {
+      const int ii = i - (TAPS - 1) + j;
+      if (ii >= 0) {
+        u[j].x += be.x; u[j].y += be.y; u[j].z += be.z; u[j].w += be.w;
+      }
+    }
+    auto tap = [](const float4& v, int j) { return j == 0 ? v.x : j == 1 ? v.y : j == 2 ? v.z : v.w; };
+    float4 y = zero4;
+#pragma unroll
+    for (int j = 0; j < TAPS; j++) {
+      y.x += tap(w[0], j) * u[j].x;
+      y.y += tap(w[1], j) * u[j].y;
+      y.z += tap(w[2], j) * u[j].z;
+      y.w += tap(w[3], j) * u[j].w;
+    }
+    *reinterpret_cast<float4*>(row + e) = y;
+    const float ss = (y.x * y.x + y.y * y.y) + (y.z * y.z + y.w * y.w);
+    if (e < nq) sq += ss;
+    else if (e < nq + nk) sk += ss;
+    if (one_token) {
+#pragma unroll
+      for (int j = 0; j < TAPS - 1; j++) *reinterpret_cast<float4*>(st + (size_t)j * C + e) = u[j + 1];
+    }
+  }
+  const float rq = qw ? 1.0f / sqrtf(block_sum256(sq, red) / (float)nq + c.eps) : 1.0f;
+  const float rk = kw ? 1.0f / sqrtf(block_sum256(sk, red) / (float)nk + c.eps) : 1.0f;
+  const size_t loc = (size_t)cache_loc[t];
+  for (int e = tid * 4; e < C; e += 1024) {      // (each thread re-reads only what it wrote)
+    float4 y = *reinterpret_cast<const float4*>(row + e);
+    if (e < nq) {
+      const float4 g = qw ? *reinterpret_cast<const float4*>(qw + e) : make_float4(1.f, 1.f, 1.f, 1.f);
+      const float r = rq * c.scale;
+      *reinterpret_cast<float4*>(q_out + (size_t)t * nq + e) = make_float4(y.x * r * g.x, y.y * r * g.y, y.z * r * g.z, y.w * r * g.w);
+    } else {
+      const bool isk = e < nq + nk;
+      if (isk) {
+        const float4 g = kw ? *reinterpret_cast<const float4*>(kw + (e - nq)) : make_float4(1.f, 1.f, 1.f, 1.f);
+        y = make_float4(y.x * rk * g.x, y.y * rk * g.y, y.z * rk * g.z, y.w * rk * g.w);
+      }
+      KT* dst = isk ? kcache + loc * nk + (e - nq) : vcache + loc * nv + (e - nq - nk);
+      if constexpr (sizeof(KT) == 2) {
+        *reinterpret_cast<uint2*>(dst) = make_uint2(ktx_pk_bf16(y.x, y.y), ktx_pk_bf16(y.z, y.w));
+      } else {
+        *reinterpret_cast<float4*>(dst) = y;
+      }
+    }
+  }
+}
+
 // the state of a causal convolution over C channels moves on behind a step: the slot's rows become the last taps - 1 inputs (this step's
 // projections + bias; older ones from the old state when the request brought fewer).  thread = channel, rows oldest first
 __global__ void __launch_bounds__(256) conv_state_update_kernel(int C, int taps, const int32_t* __restrict__ q_indptr,
@@ -1061,12 +1152,12 @@ int ktx_swa_prep(const ktx_swa_config* cfg, int T, const float* d_proj, int64_t 
   return 0;
 }
 
-int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
+int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int max_q_len, int taps, const float* d_proj, int64_t ldp, const float* d_bias,
                       const float* d_conv_w, const float* d_q_norm_w, const float* d_k_norm_w, const int32_t* d_q_indptr,
                       const int32_t* d_pos0, const int32_t* d_slot, const int32_t* d_tok_req, float* d_conv_state,
                       const int32_t* d_cache_loc, void* d_kcache, void* d_vcache, float* d_q_out, ktx_stream_t stream) {
   if (swa_check(cfg, "ktx_swa_conv_prep")) return -1;
-  KTX_REQUIRE(B >= 0 && T >= 0 && d_proj && d_q_indptr && d_pos0 && d_slot && d_tok_req && d_cache_loc && d_kcache && d_vcache && d_q_out,
+  KTX_REQUIRE(B >= 0 && T >= 0 && max_q_len >= 0 && d_proj && d_q_indptr && d_pos0 && d_slot && d_tok_req && d_cache_loc && d_kcache && d_vcache && d_q_out,
               "ktx_swa_conv_prep: null pointer");
   KTX_REQUIRE(taps >= 0 && taps <= CP_MAX_TAPS && (taps <= 1 || (d_conv_w && d_conv_state)),
               "ktx_swa_conv_prep: at most 16 taps; a convolution needs its weights and state slots");
@@ -1077,6 +1168,36 @@ int ktx_swa_conv_prep(const ktx_swa_config* cfg, int B, int T, int taps, const f
   if (T == 0 || B == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
   const size_t lds = (size_t)C * 4;
+  const int nq = cfg->heads * cfg->dim, nk = cfg->kv_heads * cfg->dim, nv = cfg->kv_heads * cfg->vdim;
+  const bool vec = taps >= 2 && taps <= 4 && nq % 4 == 0 && nk % 4 == 0 && nv % 4 == 0 && ldp % 4 == 0 && aligned16(d_proj) &&
+                   aligned16(d_conv_w) && aligned16(d_conv_state) && (!d_bias || aligned16(d_bias)) && (!d_q_norm_w || aligned16(d_q_norm_w)) &&
+                   (!d_k_norm_w || aligned16(d_k_norm_w)) && aligned16(d_q_out) && aligned16(d_kcache) && aligned16(d_vcache);
+  if (vec) {
+    const int one = max_q_len == 1 ? 1 : 0;
+#define KTX_CP_GO(KT, TAPS)                                                                                                          \
+  do {                                                                                                                               \
+    KTX_HIP(ktx_set_max_lds((const void*)swa_conv_prep_vec_kernel<KT, TAPS>, 150 * 1024));                                           \
+    swa_conv_prep_vec_kernel<KT, TAPS><<<T, 256, lds, st>>>(*cfg, d_proj, ldp, d_bias, d_conv_w, d_q_norm_w, d_k_norm_w, d_q_indptr,  \
+                                                            d_pos0, d_slot, d_tok_req, d_conv_state, one, d_cache_loc, (KT*)d_kcache, \
+                                                            (KT*)d_vcache, d_q_out);                                                 \
+  } while (0)
+#define KTX_CP_TAPS(KT)               \
+  do {                                \
+    if (taps == 2) KTX_CP_GO(KT, 2);  \
+    else if (taps == 3) KTX_CP_GO(KT, 3); \
+    else KTX_CP_GO(KT, 4);            \
+  } while (0)
+    if (cfg->cache_dtype == KTX_SEQ_F32) KTX_CP_TAPS(float);
+    else KTX_CP_TAPS(bf16_t);
+#undef KTX_CP_TAPS
+#undef KTX_CP_GO
+    KTX_HIP(hipGetLastError());
+    if (!one) {
+      conv_state_update_kernel<<<dim3((C + 255) / 256, B), 256, 0, st>>>(C, taps, d_q_indptr, d_pos0, d_slot, d_proj, ldp, d_bias, d_conv_state);
+      KTX_HIP(hipGetLastError());
+    }
+    return 0;
+  }
   if (cfg->cache_dtype == KTX_SEQ_F32) {
     KTX_HIP(ktx_set_max_lds((const void*)swa_conv_prep_kernel<float>, 150 * 1024));
     swa_conv_prep_kernel<float><<<T, 256, lds, st>>>(*cfg, taps, d_proj, ldp, d_bias, d_conv_w, d_q_norm_w, d_k_norm_w, d_q_indptr, d_pos0,
