@@ -110,7 +110,7 @@ __global__ void __launch_bounds__(256) gated_norm_add_kernel(int W, const float*
 // v = layer_norm(alpha * x + y + ybias); with a stack: level `level` of it receives v, and with dwa the row handed on is the weighted
 // sum of levels 0 .. level.  The row lives in LDS between the passes; every level's entry is requested before the sum is formed.
 template <typename OT>
-__global__ void __launch_bounds__(256) postnorm_mix_kernel(int W, const float* __restrict__ xin, float* __restrict__ xout,
+__global__ void __launch_bounds__(256) postnorm_mix_kernel(int W, const float* xin, float* xout,
                                                            ktx_postnorm_args a, OT* __restrict__ lp) {
   extern __shared__ float zrow[];
   __shared__ float red[4];
@@ -151,6 +151,88 @@ __global__ void __launch_bounds__(256) postnorm_mix_kernel(int W, const float* _
     }
     xout[ro + e] = v;
     if (lp) st_elem(lp, ro + e, v);
+  }
+}
+
+// The same update for rows of at most 256 * EPT entries, held in registers: a thread owns entries tid, tid + 256, ...; every load of
+// a phase (x, y and the bias; then the norm's weights and the lower levels of the stack) is requested before the first is used, so a
+// one-row launch (a decode step) costs a few memory round trips instead of one per entry.
+template <typename OT, int EPT>
+__global__ void __launch_bounds__(256) postnorm_mix_reg_kernel(int W, const float* xin, float* xout,
+                                                               ktx_postnorm_args a, OT* __restrict__ lp) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const size_t ro = (size_t)t * W;
+  float z[EPT], yv[EPT], bv[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; i++) {
+    const int e = tid + i * 256;
+    const bool in = e < W;
+    z[i] = in ? xin[ro + e] : 0.f;
+    yv[i] = in && a.y ? a.y[(size_t)t * a.ldy + e] : 0.f;
+    bv[i] = in && a.ybias ? a.ybias[e] : 0.f;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < EPT; i++) {
+    z[i] = (a.alpha * z[i] + yv[i]) + bv[i];
+    s += z[i];                                   // (entries beyond W are 0)
+  }
+  const int lv = a.level;
+  const bool avg = a.stack && a.dwa;
+  // the norm's weights and the first lower levels of the stack are on their way while the row is reduced
+  float wv[EPT], lo[EPT];
+#pragma unroll
+  for (int i = 0; i < EPT; i++) {
+    const int e = tid + i * 256;
+    const bool in = e < W;
+    wv[i] = in ? a.w[e] : 0.f;
+    bv[i] = in && a.b ? a.b[e] : 0.f;
+    lo[i] = in && avg && lv > 0 ? a.stack[ro + e] : 0.f;
+  }
+  const float mean = block_sum256(s, red) / (float)W;
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < EPT; i++) {
+    const float d = tid + i * 256 < W ? z[i] - mean : 0.f;
+    q += d * d;
+  }
+  const float r = 1.0f / sqrtf(block_sum256(q, red) / (float)W + a.eps);
+#pragma unroll
+  for (int i = 0; i < EPT; i++) z[i] = (z[i] - mean) * r * wv[i] + bv[i];
+  if (a.stack) {
+#pragma unroll
+    for (int i = 0; i < EPT; i++) {
+      const int e = tid + i * 256;
+      if (e < W) a.stack[(size_t)lv * a.stack_stride + ro + e] = z[i];
+    }
+  }
+  if (avg) {
+    const float wl = a.dwa[lv];
+#pragma unroll
+    for (int i = 0; i < EPT; i++) z[i] *= wl;
+    for (int j = 0; j < lv; j++) {               // level j is in `lo`; level j + 1 is requested before it is used
+      const float wj = a.dwa[j];
+      float nx[EPT];
+#pragma unroll
+      for (int i = 0; i < EPT; i++) {
+        const int e = tid + i * 256;
+        nx[i] = e < W && j + 1 < lv ? a.stack[(size_t)(j + 1) * a.stack_stride + ro + e] : 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < EPT; i++) {
+        z[i] += wj * lo[i];
+        lo[i] = nx[i];
+      }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < EPT; i++) {
+    const int e = tid + i * 256;
+    if (e < W) {
+      xout[ro + e] = z[i];
+      if (lp) st_elem(lp, ro + e, z[i]);
+    }
   }
 }
 
@@ -1176,6 +1258,20 @@ int ktx_postnorm_mix(int T, int W, const float* d_x_in, float* d_x_out, const kt
   KTX_REQUIRE((size_t)W * 4 <= 150 * 1024, "ktx_postnorm_mix: a row must fit the LDS");
   if (T == 0) return 0;
   hipStream_t st = (hipStream_t)stream;
+  const bool lp16 = a->out_lp && a->out_dtype == KTX_SEQ_BF16;
+  if (W <= 256 * 16) {
+#define KTX_PN_GO(EPT)                                                                                                    \
+  do {                                                                                                                    \
+    if (lp16) postnorm_mix_reg_kernel<bf16_t, EPT><<<T, 256, 0, st>>>(W, d_x_in, d_x_out, *a, (bf16_t*)a->out_lp);        \
+    else postnorm_mix_reg_kernel<float, EPT><<<T, 256, 0, st>>>(W, d_x_in, d_x_out, *a, (float*)a->out_lp);               \
+  } while (0)
+    if (W <= 256 * 4) KTX_PN_GO(4);
+    else if (W <= 256 * 8) KTX_PN_GO(8);
+    else KTX_PN_GO(16);
+#undef KTX_PN_GO
+    KTX_HIP(hipGetLastError());
+    return 0;
+  }
   if (a->out_lp && a->out_dtype == KTX_SEQ_BF16) {
     KTX_HIP(ktx_set_max_lds((const void*)postnorm_mix_kernel<bf16_t>, 150 * 1024));
     postnorm_mix_kernel<bf16_t><<<T, 256, (size_t)W * 4, st>>>(W, d_x_in, d_x_out, *a, (bf16_t*)a->out_lp);

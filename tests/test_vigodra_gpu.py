@@ -66,10 +66,11 @@ def batch_of(cache, entries):
 
 
 # ---- the element-wise kernels and the norm ---------------------------------------------------------------------------------------
-@pytest.mark.parametrize("W,levels,lp", [(32, 0, None), (48, 1, BF16), (260, 4, BF16), (1024, 11, F32), (7, 3, None)])
+@pytest.mark.parametrize("W,levels,lp", [(32, 0, None), (48, 1, BF16), (260, 4, BF16), (1024, 11, F32), (7, 3, None), (1500, 2, BF16),
+                                         (4096, 3, None), (4100, 2, BF16)])
 def test_post_norm_with_scaled_residual_and_depth_average(W, levels, lp):
     """ktx_postnorm_mix against the plain layer norm and weighted sum: with and without the sublayer's output, its bias, the stack and the
-    average; in place and out of place; a low-precision copy."""
+    average; in place and out of place; a low-precision copy; rows held in registers (up to 4096 entries) and in LDS (beyond)."""
     from ktransformers_amd._native_hyb import postnorm_mix
     g = torch.Generator().manual_seed(W + levels)
     T, alpha, eps = 5, 2.25, 1e-5
