@@ -2206,9 +2206,13 @@ class VigKernelTimer(SwaKernelTimer):
     """HIP events around every binding a Vigodra step calls."""
     HYB = ("layer_norm", "postnorm_mix", "glu_clamp_rows", "sigmoid_gate_rows", "latattn_prep", "latattn_forward", "latattn_mfma", "head_gemm")
     SWA = ("swa_conv_prep", "swa_forward", "swa_mfma")
+    SEQ = ("embed_rows", "dense_gemm", "dense_gemv_glu")
 
     def _cost(self, name, a, kw, out):
         nb = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else 0
+        if name == "dense_gemv_glu":
+            M, K = a[0].shape
+            return "dense_gemm M=decode", 2.0 * M * a[1].shape[0] * K, M * K * a[0].element_size() + nb(a[1]) + nb(out)
         if name == "postnorm_mix":
             x = a[0]
             levels = (kw.get("level", 0) + 1) if kw.get("dwa") is not None else (1 if kw.get("stack") is not None else 0)

@@ -69,11 +69,11 @@ int ktx_poly_norm(int T, int F, const float* d_z, int64_t ldz, const float* d_bi
 /* out[r][f] = silu(in[r][f]) * in[r][F + f]: fp32 rows of 2F (stride ldi) -> [R][F] of out_dtype. */
 int ktx_silu_mul_rows(int R, int F, const float* d_in, int64_t ldi, void* d_out, int out_dtype, ktx_stream_t stream);
 
-/* out[r][f] = g * sigmoid(slope * g) * (u + up_shift) with g = min(in[r][f], limit), u = clamp(in[r][F + f], -limit, limit): the
- * activation of a GLU whose gate is capped from above and whose linear half is clamped (limit = INFINITY: neither); fp32 rows of 2F
- * (stride ldi) -> [R][F] of out_dtype. */
-int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, void* d_out, int out_dtype,
-                       ktx_stream_t stream);
+/* out[r][f] = g * sigmoid(slope * g) * (u + up_shift) with g = min(gate, limit), u = clamp(up, -limit, limit): the activation of a GLU
+ * whose gate is capped from above and whose linear half is clamped (limit = INFINITY: neither); fp32 rows of 2F (stride ldi) holding
+ * gate = in[r][f], up = in[r][F + f], or — paired != 0 — gate = in[r][2f], up = in[r][2f + 1]; -> [R][F] of out_dtype. */
+int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, int paired, void* d_out,
+                       int out_dtype, ktx_stream_t stream);
 
 /* out[r][c] = o[r][c] * sigmoid(gate[r][c]): o [R][N] of o_dtype, gate fp32 rows of stride ldg -> [R][N] of out_dtype (an output gate
  * on an attention's concatenated heads). */

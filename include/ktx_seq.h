@@ -32,6 +32,12 @@ enum { KTX_ACT_NONE = 0, KTX_ACT_GELU_TANH = 1 };
 int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const int32_t* d_pos, const void* d_embed,
                      int embed_dtype, const double* d_inv_freq, float* d_x, ktx_stream_t stream);
 
+/* The gate | up product of a GLU and its activation in one launch, for steps of at most 16 rows: W bf16 [2F][K] with rows ALTERNATING
+ * gate_f, up_f;  Y[m][f] = g sigmoid(slope g) (u + up_shift), g = min(gate_f . A[m], limit), u = clamp(up_f . A[m], -limit, limit)
+ * (limit = INFINITY: unbounded).  K a multiple of 32, 16-byte aligned rows; A fp32 or bf16 (rounded to bf16 on the way in), Y fp32 or bf16. */
+int ktx_dense_gemv_glu(int M, int F, int K, const void* d_A, int a_dtype, int64_t lda, const void* d_W, void* d_Y, int y_dtype, int64_t ldy,
+                       float limit, float slope, float up_shift, ktx_stream_t stream);
+
 /* Y[m][n] = act(sum_k A[m][k] * W[n][k]), any M, N, K >= 1.  The product runs in W's type: bf16 MFMA with fp32 accumulation
  * (A rounded to bf16 on the way in when it is fp32) or fp32 MFMA (A must be fp32).  Y is fp32 or bf16.  lda / ldy in elements.
  * ksplit > 1 splits K over ksplit workgroups per tile that add into a ZEROED fp32 Y with atomics (small M; act must be NONE). */

@@ -37,7 +37,7 @@ lib.ktx_gated_norm_add.argtypes = [_I, _I, _P, _L, _P, _P, _P, _P, _I, _P, _L, _
 lib.ktx_poly_norm.argtypes = [_I, _I, _P, _L, _P, _P, _F, _P, _I, _P]
 lib.ktx_silu_mul_rows.argtypes = [_I, _I, _P, _L, _P, _I, _P]
 lib.ktx_postnorm_mix.argtypes = [_I, _I, _P, _P, C.POINTER(_PostNormArgs), _P]
-lib.ktx_glu_clamp_rows.argtypes = [_I, _I, _P, _L, _F, _F, _F, _P, _I, _P]
+lib.ktx_glu_clamp_rows.argtypes = [_I, _I, _P, _L, _F, _F, _F, _I, _P, _I, _P]
 lib.ktx_sigmoid_gate_rows.argtypes = [_I, _I, _P, _I, _P, _L, _P, _I, _P]
 lib.ktx_head_gate_norm.argtypes = [_I, _I, _I, _F, _P, _P, _L, _P, _I, _I, _P, _I, _P]
 lib.ktx_delta_prep.argtypes = [C.POINTER(_DeltaConfig), _I, _I, _P, _P, _P, _P, _P, _L, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _P]
@@ -175,14 +175,15 @@ def postnorm_mix(x_in: torch.Tensor, x_out: torch.Tensor, w: torch.Tensor, b: to
     return x_out if lp is None else lp
 
 
-def glu_clamp_rows(gu: torch.Tensor, limit: float | None, slope: float = 1.0, up_shift: float = 0.0, out_dtype=torch.float32) -> torch.Tensor:
-    """[R, 2F] (gate | up) -> g * sigmoid(slope * g) * (u + up_shift), g = min(gate, limit), u = clamp(up, -limit, limit); [R, F]
-    (ktx_glu_clamp_rows; limit None: neither is bounded)."""
+def glu_clamp_rows(gu: torch.Tensor, limit: float | None, slope: float = 1.0, up_shift: float = 0.0, out_dtype=torch.float32,
+                   paired: bool = False) -> torch.Tensor:
+    """[R, 2F] (gate | up; paired: gate_0, up_0, gate_1, up_1, ...) -> g * sigmoid(slope * g) * (u + up_shift), g = min(gate, limit),
+    u = clamp(up, -limit, limit); [R, F] (ktx_glu_clamp_rows; limit None: neither is bounded)."""
     p, ld = _rows_f32(gu, "glu_clamp_rows")
     R, F = gu.shape[0], gu.shape[1] // 2
     out = torch.empty((R, F), dtype=out_dtype, device=gu.device)
     check(lib.ktx_glu_clamp_rows(R, F, p, ld, float("inf") if limit is None else float(limit), float(slope), float(up_shift),
-                                 out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(gu.device)))
+                                 1 if paired else 0, out.data_ptr(), SEQ_DTYPE[out_dtype], _stream_ptr(gu.device)))
     return out
 
 

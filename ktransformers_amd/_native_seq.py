@@ -44,6 +44,9 @@ def _load() -> C.CDLL:
     lib.ktx_embed_sinpos.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     lib.ktx_dense_gemm.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_int, C.c_void_p, C.c_int,
                                    C.c_int64, C.c_int, C.c_int, C.c_void_p]
+    if hasattr(lib, "ktx_dense_gemv_glu"):
+        lib.ktx_dense_gemv_glu.argtypes = [C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int64, C.c_void_p, C.c_void_p, C.c_int, C.c_int64,
+                                           C.c_float, C.c_float, C.c_float, C.c_void_p]
     lib.ktx_sigattn_prep.argtypes = [C.POINTER(_SigAttnConfig), C.c_int, C.c_void_p, C.c_int64, C.c_int, C.c_int, C.c_void_p, C.c_void_p,
                                      C.c_float] + [C.c_void_p] * 6
     lib.ktx_sigattn_forward.argtypes = [C.POINTER(_SigAttnConfig), C.c_int] + [C.c_void_p] * 9 + [C.c_int, C.c_void_p, C.c_void_p, C.c_int,
@@ -133,6 +136,28 @@ def dense_gemm(a: torch.Tensor, w: torch.Tensor, out_dtype=torch.float32, act: s
         raise KtxError("dense_gemm: out does not fit")
     check(lib.ktx_dense_gemm(M, N, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), w.data_ptr(), SEQ_DTYPE[w.dtype], out.data_ptr(),
                              SEQ_DTYPE[out_dtype], out.stride(0), ACT[act], int(ksplit), _stream_ptr(a.device)))
+    return out
+
+
+GEMV_GLU_MAX_M = 16
+
+
+def dense_gemv_glu_eligible(a: torch.Tensor, w: torch.Tensor) -> bool:
+    return (a.dim() == 2 and a.shape[0] <= GEMV_GLU_MAX_M and w.dtype == torch.bfloat16 and a.dtype in SEQ_DTYPE and a.shape[1] % 32 == 0
+            and a.stride(1) == 1 and (a.stride(0) * a.element_size()) % 16 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0)
+
+
+def dense_gemv_glu(a: torch.Tensor, w_pairs: torch.Tensor, limit: float | None, slope: float, up_shift: float, out_dtype=torch.float32) -> torch.Tensor:
+    """Decode-sized GLU front half in one launch (ktx_dense_gemv_glu): a [M <= 16, K] x w_pairs [2F, K] (bf16, rows alternating gate_f,
+    up_f) -> g sigmoid(slope g) (u + up_shift) with the bounded g, u; [M, F] of out_dtype."""
+    if not dense_gemv_glu_eligible(a, w_pairs) or not w_pairs.is_contiguous() or w_pairs.shape[1] != a.shape[1] or w_pairs.shape[0] % 2:
+        raise KtxError(f"dense_gemv_glu: {a.dtype} {tuple(a.shape)} x {w_pairs.dtype} {tuple(w_pairs.shape)}^T does not fit")
+    M, K = a.shape
+    Fh = w_pairs.shape[0] // 2
+    out = torch.empty((M, Fh), dtype=out_dtype, device=a.device)
+    check(lib.ktx_dense_gemv_glu(M, Fh, K, a.data_ptr(), SEQ_DTYPE[a.dtype], a.stride(0), w_pairs.data_ptr(), out.data_ptr(), SEQ_DTYPE[out_dtype],
+                                 out.stride(0), float("inf") if limit is None else float(limit), float(slope), float(up_shift),
+                                 _stream_ptr(a.device)))
     return out
 
 

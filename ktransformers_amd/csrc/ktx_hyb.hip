@@ -259,15 +259,17 @@ __global__ void __launch_bounds__(256) poly_norm_kernel(int F, const float* __re
   }
 }
 
-// out[r][f] = g * sigmoid(slope * g) * (u + up_shift), g = min(in[r][f], limit), u = clamp(in[r][F + f], -limit, limit)
+// out[r][f] = g * sigmoid(slope * g) * (u + up_shift), g = min(gate, limit), u = clamp(up, -limit, limit); (gate, up) = in[r][f],
+// in[r][F + f], or — paired — in[r][2f], in[r][2f + 1]
 template <typename OT>
 __global__ void __launch_bounds__(256) glu_clamp_rows_kernel(size_t n, int F, const float* __restrict__ in, int64_t ldi, float limit,
-                                                             float slope, float up_shift, OT* __restrict__ out) {
+                                                             float slope, float up_shift, int paired, OT* __restrict__ out) {
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i >= n) return;
   const size_t r = i / F;
   const int f = (int)(i % F);
-  const float g = fminf(in[r * ldi + f], limit), u = fminf(fmaxf(in[r * ldi + F + f], -limit), limit);
+  const float gv = paired ? in[r * ldi + 2 * f] : in[r * ldi + f], uv = paired ? in[r * ldi + 2 * f + 1] : in[r * ldi + F + f];
+  const float g = fminf(gv, limit), u = fminf(fmaxf(uv, -limit), limit);
   st_elem(out, i, g * sigmoid_f32(slope * g) * (u + up_shift));
 }
 
@@ -1283,16 +1285,16 @@ int ktx_postnorm_mix(int T, int W, const float* d_x_in, float* d_x_out, const kt
   return 0;
 }
 
-int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, void* d_out, int out_dtype,
-                       ktx_stream_t stream) {
+int ktx_glu_clamp_rows(int R, int F, const float* d_in, int64_t ldi, float limit, float slope, float up_shift, int paired, void* d_out,
+                       int out_dtype, ktx_stream_t stream) {
   KTX_REQUIRE(R >= 0 && F > 0 && d_in && d_out && dtype_ok(out_dtype) && ldi >= 2 * (int64_t)F && limit > 0.f, "ktx_glu_clamp_rows: arguments");
   if (R == 0) return 0;
   const size_t n = (size_t)R * F;
   hipStream_t st = (hipStream_t)stream;
   if (out_dtype == KTX_SEQ_F32)
-    glu_clamp_rows_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, (float*)d_out);
+    glu_clamp_rows_kernel<float><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, paired, (float*)d_out);
   else
-    glu_clamp_rows_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, (bf16_t*)d_out);
+    glu_clamp_rows_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(n, F, d_in, ldi, limit, slope, up_shift, paired, (bf16_t*)d_out);
   KTX_HIP(hipGetLastError());
   return 0;
 }

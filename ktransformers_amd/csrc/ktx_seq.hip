@@ -739,9 +739,12 @@ __global__ void __launch_bounds__(256) dense_gemv_kernel(int M, int N, int K, co
 // decode-sized GEMM on the matrix cores (M <= 16, bf16 weights, K % 32 == 0): workgroup = 16 weight rows, its four wavefronts take a
 // quarter of K each; a lane streams ITS weight row's 16-byte pieces straight from memory into the B operand (no LDS on the weight
 // path), the activation rows (few, L2-resident) fill the A operand; partial tiles meet in LDS.
-template <typename AT, typename YT>
+// GLU: W's rows alternate gate_f, up_f (N = 2F); neighbouring lanes hold a pair's two products and the even one writes
+// Y[m][f] = g sigmoid(slope g) (u + shift), g = min(gate, limit), u = clamp(up, -limit, limit).
+template <typename AT, typename YT, bool GLU>
 __global__ void __launch_bounds__(256) dense_gemv_mfma_kernel(int M, int N, int K, const AT* __restrict__ A, int64_t lda,
-                                                              const bf16_t* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act) {
+                                                              const bf16_t* __restrict__ W, YT* __restrict__ Y, int64_t ldy, int act,
+                                                              float limit, float slope, float shift) {
   __shared__ float red[4][64][4];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l16 = lane & 15, lq = lane >> 4;
   const int n = blockIdx.x * 16 + l16;
@@ -769,12 +772,18 @@ __global__ void __launch_bounds__(256) dense_gemv_mfma_kernel(int M, int N, int 
 #pragma unroll
   for (int r = 0; r < 4; r++) red[wave][lane][r] = acc[r];
   __syncthreads();
-  if (wave == 0 && wok) {
+  if (wave == 0) {
 #pragma unroll
     for (int r = 0; r < 4; r++) {
       const int m = lq * 4 + r;
-      if (m < M) {
-        float v = ((red[0][lane][r] + red[1][lane][r]) + red[2][lane][r]) + red[3][lane][r];
+      float v = ((red[0][lane][r] + red[1][lane][r]) + red[2][lane][r]) + red[3][lane][r];
+      if constexpr (GLU) {
+        const float other = __shfl_xor(v, 1);      // (N is even: a pair is inside or outside together)
+        if (wok && m < M && (l16 & 1) == 0) {
+          const float g = fminf(v, limit), u = fminf(fmaxf(other, -limit), limit);
+          st_elem(Y, (size_t)m * ldy + (n >> 1), g * sigmoid_f32(slope * g) * (u + shift));
+        }
+      } else if (wok && m < M) {
         if (act == KTX_ACT_GELU_TANH) v = gelu_tanh_f32(v);
         st_elem(Y, (size_t)m * ldy + n, v);
       }
@@ -1177,6 +1186,29 @@ int ktx_embed_sinpos(int T, int width, int vocab, const int32_t* d_tokens, const
   return 0;
 }
 
+int ktx_dense_gemv_glu(int M, int F, int K, const void* d_A, int a_dtype, int64_t lda, const void* d_W, void* d_Y, int y_dtype, int64_t ldy,
+                       float limit, float slope, float up_shift, ktx_stream_t stream) {
+  KTX_REQUIRE(M >= 0 && M <= 16 && F > 0 && K > 0 && K % 32 == 0 && d_A && d_W && d_Y && lda >= K && ldy >= F && limit > 0.f,
+              "ktx_dense_gemv_glu: at most 16 rows, K a multiple of 32");
+  KTX_REQUIRE((a_dtype == KTX_SEQ_F32 || a_dtype == KTX_SEQ_BF16) && (y_dtype == KTX_SEQ_F32 || y_dtype == KTX_SEQ_BF16),
+              "ktx_dense_gemv_glu: unknown element type");
+  KTX_REQUIRE(aligned16(d_W) && aligned16(d_A) && (lda * (a_dtype == KTX_SEQ_F32 ? 4 : 2)) % 16 == 0, "ktx_dense_gemv_glu: 16-byte aligned rows");
+  if (M == 0) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const int N = 2 * F;
+  const unsigned blocks = (unsigned)((N + 15) / 16);
+#define KTX_GLU_GO(AT, YT)                                                                                                         \
+  dense_gemv_mfma_kernel<AT, YT, true><<<blocks, 256, 0, st>>>(M, N, K, (const AT*)d_A, lda, (const bf16_t*)d_W, (YT*)d_Y, ldy, 0, limit, \
+                                                               slope, up_shift)
+  if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32) KTX_GLU_GO(float, float);
+  else if (a_dtype == KTX_SEQ_F32) KTX_GLU_GO(float, bf16_t);
+  else if (y_dtype == KTX_SEQ_F32) KTX_GLU_GO(bf16_t, float);
+  else KTX_GLU_GO(bf16_t, bf16_t);
+#undef KTX_GLU_GO
+  KTX_HIP(hipGetLastError());
+  return 0;
+}
+
 int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t lda, const void* d_W, int w_dtype, void* d_Y,
                    int y_dtype, int64_t ldy, int act, int ksplit, ktx_stream_t stream) {
   KTX_REQUIRE(M >= 0 && N > 0 && K > 0, "ktx_dense_gemm: M >= 0, N, K > 0");
@@ -1192,13 +1224,13 @@ int ktx_dense_gemm(int M, int N, int K, const void* d_A, int a_dtype, int64_t ld
       (lda * (a_dtype == KTX_SEQ_F32 ? 4 : 2)) % 16 == 0) {
     const unsigned blocks = (unsigned)((N + 15) / 16);
     if (a_dtype == KTX_SEQ_F32 && y_dtype == KTX_SEQ_F32)
-      dense_gemv_mfma_kernel<float, float><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act);
+      dense_gemv_mfma_kernel<float, float, false><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act, 0.f, 0.f, 0.f);
     else if (a_dtype == KTX_SEQ_F32)
-      dense_gemv_mfma_kernel<float, bf16_t><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act);
+      dense_gemv_mfma_kernel<float, bf16_t, false><<<blocks, 256, 0, st>>>(M, N, K, (const float*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act, 0.f, 0.f, 0.f);
     else if (y_dtype == KTX_SEQ_F32)
-      dense_gemv_mfma_kernel<bf16_t, float><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act);
+      dense_gemv_mfma_kernel<bf16_t, float, false><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (float*)d_Y, ldy, act, 0.f, 0.f, 0.f);
     else
-      dense_gemv_mfma_kernel<bf16_t, bf16_t><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act);
+      dense_gemv_mfma_kernel<bf16_t, bf16_t, false><<<blocks, 256, 0, st>>>(M, N, K, (const bf16_t*)d_A, lda, (const bf16_t*)d_W, (bf16_t*)d_Y, ldy, act, 0.f, 0.f, 0.f);
     KTX_HIP(hipGetLastError());
     return 0;
   }

@@ -174,7 +174,9 @@ class KPolyNormMLP(BaseInjectedModule):
 class KClampedGLUMLP(BaseInjectedModule):
     """Three-matrix gated feed-forward on an fp32 residual stream whose halves are bounded before they meet:
     W_down (g sigmoid(slope g) (u + up_shift)), g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit).  gate and up are one product
-    ([gate ; up] merged at load), the activation one launch (include/ktx_hyb.h `ktx_glu_clamp_rows`), fp32 out.  limit (None: unbounded),
+    (merged at load with their rows ALTERNATING, so a pair's two products meet in neighbouring lanes): for decode-sized steps product and
+    activation are one launch (include/ktx_seq.h `ktx_dense_gemv_glu`), otherwise the activation follows the product
+    (include/ktx_hyb.h `ktx_glu_clamp_rows`, paired form); fp32 out.  limit (None: unbounded),
     slope and up_shift are read from the replaced module.  Checkpoint tensors: `<key>.gate`, `<key>.up` [ff, width], `<key>.down`
     [width, ff]."""
 
@@ -191,11 +193,14 @@ class KClampedGLUMLP(BaseInjectedModule):
         gate, up, down = get("gate"), get("up"), get("down")
         if tuple(gate.shape) != (self.ff, self.width) or tuple(up.shape) != (self.ff, self.width) or tuple(down.shape) != (self.width, self.ff):
             raise ValueError(f"{self.key}: tensor shapes do not fit ff={self.ff} width={self.width}")
-        self.w.update(gate_up=torch.cat([gate, up]).contiguous(), down=down.contiguous())
+        self.w.update(gate_up=torch.stack([gate, up], dim=1).reshape(2 * self.ff, self.width).contiguous(), down=down.contiguous())
 
     def forward(self, h: torch.Tensor) -> torch.Tensor:
         """h [T, width] in the compute type -> fp32 [T, width]."""
         from ktransformers_amd._native_hyb import glu_clamp_rows
-        from ktransformers_amd._native_seq import dense_gemm
-        a = glu_clamp_rows(dense_gemm(h, self.w["gate_up"]), self.limit, self.slope, self.up_shift, out_dtype=self.compute_dtype)
+        from ktransformers_amd._native_seq import dense_gemm, dense_gemv_glu, dense_gemv_glu_eligible
+        if dense_gemv_glu_eligible(h, self.w["gate_up"]):
+            a = dense_gemv_glu(h, self.w["gate_up"], self.limit, self.slope, self.up_shift, out_dtype=self.compute_dtype)
+        else:
+            a = glu_clamp_rows(dense_gemm(h, self.w["gate_up"]), self.limit, self.slope, self.up_shift, out_dtype=self.compute_dtype, paired=True)
         return dense_gemm(a, self.w["down"])

@@ -121,10 +121,31 @@ def test_bounded_glu_activation_and_sigmoid_gate(limit, dtype):
     want = gate * torch.sigmoid(1.702 * gate) * (up + 1.0)
     got = glu_clamp_rows(gu.to(DEV), limit, 1.702, 1.0, out_dtype=dtype)
     assert rel(got, want) < (1e-6 if dtype == F32 else 4e-3)
+    pairs = torch.stack([gu[:, :37], gu[:, 37:]], dim=2).reshape(9, 74)          # gate_0, up_0, gate_1, up_1, ...
+    got = glu_clamp_rows(pairs.to(DEV), limit, 1.702, 1.0, out_dtype=dtype, paired=True)
+    assert rel(got, want) < (1e-6 if dtype == F32 else 4e-3)
     wide = torch.randn(9, 100, generator=g)
     o = torch.randn(9, 37, generator=g).to(dtype)
     got = sigmoid_gate_rows(o.to(DEV), wide.to(DEV)[:, 11:48], out_dtype=dtype)
     assert rel(got, o.double() * torch.sigmoid(wide[:, 11:48].double())) < (1e-6 if dtype == F32 else 4e-3)
+
+
+@pytest.mark.parametrize("M,F,K,limit", [(1, 40, 64, 1.5), (8, 37, 96, None), (16, 16, 32, 0.5), (3, 300, 2048, 7.0)])
+@pytest.mark.parametrize("a_dtype,out_dtype", [(F32, F32), (BF16, BF16), (F32, BF16)])
+def test_decode_sized_glu_product_with_the_activation_in_its_launch(M, F, K, limit, a_dtype, out_dtype):
+    from ktransformers_amd._native_seq import dense_gemv_glu, dense_gemv_glu_eligible
+    g = torch.Generator().manual_seed(M + F)
+    a = torch.randn(M, K, generator=g).to(BF16)
+    gate, up = (torch.randn(F, K, generator=g) * 2 / math.sqrt(K)).to(BF16), (torch.randn(F, K, generator=g) * 2 / math.sqrt(K)).to(BF16)
+    gv, uv = a.double() @ gate.double().T, a.double() @ up.double().T
+    if limit is not None:
+        gv, uv = gv.clamp(max=limit), uv.clamp(-limit, limit)
+    want = gv * torch.sigmoid(1.702 * gv) * (uv + 1.0)
+    w = torch.stack([gate, up], dim=1).reshape(2 * F, K).contiguous().to(DEV)
+    ad = a.to(a_dtype).to(DEV)
+    assert dense_gemv_glu_eligible(ad, w) and not dense_gemv_glu_eligible(torch.zeros(17, K, dtype=a_dtype, device=DEV), w)
+    got = dense_gemv_glu(ad, w, limit, 1.702, 1.0, out_dtype=out_dtype)
+    assert rel(got, want) < (2e-5 if out_dtype == F32 else 4e-3)
 
 
 def test_distance_rows_follow_the_plain_bucket_rule():
