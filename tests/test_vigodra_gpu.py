@@ -3,7 +3,6 @@ kernels and operator, then the model through the framework's registry, cache man
 prompts, token-by-token decoding, portions, unequal batches, reused pages and slots, keys at the window's edge, among the kept first
 tokens and at page borders, odd sizes.  Small random configurations; fp32 runs are held to rounding, bf16 runs to bf16 rounding."""
 import math
-from types import SimpleNamespace
 
 import pytest
 import torch
@@ -157,10 +156,6 @@ def test_distance_rows_follow_the_plain_bucket_rule():
 
 
 # ---- attention kernels with hand-made queries, keys and values: one key made to stand out -----------------------------------------
-def paged(cache, batch_entries):
-    return batch_of(cache, batch_entries)
-
-
 def run_swa(H, G, D, V, T, window, keep, rel_t, far, sink, q, k, v, dtype, kernel, nsplit=1, page_size=8, t_new=None):
     """The attention kernels on keys and values written straight into paged caches; the last t_new positions are the queries."""
     from ktransformers_amd._native_swa import swa_config, swa_forward, swa_mfma, swa_mfma_eligible
