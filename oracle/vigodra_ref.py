@@ -127,6 +127,18 @@ def latent_rows(P, pre, c, h, eps):
     return lat, kr
 
 
+def latent_core(q_lat, rows, rank, scale, size=None):
+    """The latent attention with the key product moved to the query side: q_lat [T, H, rank + rot] against the cached rows [T, rank + rot]
+    (latent | rotated key part) of ONE sequence -> each head's softmax-weighted sum of the LATENTS [T, H, rank] (W_uv follows)."""
+    T, H, _ = q_lat.shape
+    see = visible_matrix(T, size, 0)
+    out = torch.zeros(T, H, rank, dtype=q_lat.dtype)
+    for hd in range(H):
+        s = (q_lat[:, hd] @ rows.T) * scale
+        out[:, hd] = torch.softmax(s.masked_fill(~see, float("-inf")), dim=1) @ rows[:, :rank]
+    return out
+
+
 def gated_latent_attention(P, pre, c, h, eps, shared=None):
     """Latent attention: keys and values of every head are products of one cached latent (plus one rotated key part all heads share);
     sliding window, ordinary softmax, heads multiplied by sigmoid(W_g h) before W_o.  `shared`: (latent, rotated key part) of the layer

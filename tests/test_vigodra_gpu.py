@@ -262,6 +262,58 @@ def test_distance_bias_decides_between_equal_keys(kernel, dtype):
             assert rel(got.view(t_new, H, V), want[T - t_new:]) < (2e-5 if kernel == "valu" else 1.5e-2), row
 
 
+def run_latent(H, L, R, T, window, scale, q, rows, dtype, kernel, nsplit=1, page_size=8, t_new=None):
+    """The latent-attention kernels (no sink) on rows written straight into a paged cache; the last t_new positions are the queries."""
+    from ktransformers_amd._native_hyb import latattn_config, latattn_forward, latattn_mfma, latattn_mfma_eligible
+    from ktransformers_amd.models.custom_cache import KHybridCache
+    cache = KHybridCache([{"latent": L + R}], 4 * T + 64, max_requests=4, page_size=page_size, dtype=dtype, device=DEV)
+    cache.admit("pad"), cache.plan([("pad", page_size + 3)])
+    t_new = T if t_new is None else t_new
+    cache.admit("r")
+    if T > t_new:
+        cache.plan([("r", T - t_new)])
+    b = cache.plan([("r", t_new)])
+    pages = cache.requests["r"]["pages"]
+    loc = torch.tensor([pages[p // page_size] * page_size + p % page_size for p in range(T)], device=DEV)
+    cache.lat_caches[0][loc] = rows.to(DEV).to(dtype)
+    cfg = latattn_config(H, 8, R, 8, L, 0, scale, window or 0, 1e-6, page_size, dtype)
+    qn = q[T - t_new:].reshape(t_new, H * (L + R)).float().contiguous().to(DEV)
+    if kernel == "mfma":
+        assert latattn_mfma_eligible(cfg)
+        return latattn_mfma(cfg, qn, cache.lat_caches[0], b, None, nsplit=nsplit, out_dtype=F32)
+    return latattn_forward(cfg, qn, cache.lat_caches[0], b, None, nsplit=nsplit, out_dtype=F32)
+
+
+@pytest.mark.parametrize("kernel,dtype,L,Rd", [("valu", F32, 24, 6), ("valu", BF16, 9, 4), ("mfma", BF16, 64, 16)])
+@pytest.mark.parametrize("nsplit", [1, 3])
+def test_latent_attention_without_a_sink_and_its_window_edge(kernel, dtype, L, Rd, nsplit):
+    """An ordinary softmax over the window (no extra term in the denominator): random rows, then ONE boosted row just inside and just
+    outside the window, at position 0 and on either side of a page border — as prompts, single decode tokens and portions of two."""
+    H, T, window, ps = 3, 77, 20, 8
+    g = torch.Generator().manual_seed(L)
+    q = (torch.randn(T, H, L + Rd, generator=g) * (L + Rd) ** -0.5).to(dtype).double()
+    rows = torch.randn(T, L + Rd, generator=g).to(dtype).double()
+    tol = 2e-5 if kernel == "valu" else 1.5e-2
+    want = R.latent_core(q, rows, L, 1.0, window)
+    for t_new in (T, 1, 2):
+        got = run_latent(H, L, Rd, T, window, 1.0, q, rows, dtype, kernel, nsplit=nsplit, page_size=ps, t_new=t_new)
+        assert rel(got.view(t_new, H, L), want[T - t_new:]) < tol, t_new
+    i = T - 1
+    for j, seen in ((i - window + 1, True), (i - window, False), (0, False), (i, True), (i - 13, True), (i - 12, True)):
+        qb, rb = q.clone() * 0.05, rows.clone()
+        rb[:, 2] *= 0.05
+        qb[i, :, :] = 0.0
+        qb[i, :, 2] = 6.0
+        rb[j, 2] = 6.0                                          # score 36 against ~0 elsewhere
+        qb, rb = qb.to(dtype).double(), rb.to(dtype).double()
+        want = R.latent_core(qb, rb, L, 1.0, window)
+        assert (float((want[i, 0] - rb[j, :L]).abs().max()) < 1e-6) == seen, j
+        for t_new in (T, 1, 2):
+            got = run_latent(H, L, Rd, T, window, 1.0, qb, rb, dtype, kernel, nsplit=nsplit, page_size=ps, t_new=t_new)
+            assert rel(got.view(t_new, H, L), want[T - t_new:]) < tol, (j, t_new)
+            assert (float((got.view(t_new, H, L)[-1, 0].double().cpu() - rb[j, :L]).abs().max()) < 3e-2) == seen, (j, t_new)
+
+
 # ---- the attention operators alone (a one-layer model without feed-forward reads its mixer's input from the embedding) -------------
 def mixer_alone(layer, dtype, seed, T=40, width=32, **kw):
     """The layer's mixer through the model: logits of a one-layer model whole, token by token and in portions, against the statement."""
