@@ -1,6 +1,8 @@
 /* ktx_swa.h — C ABI of the kernels (libktx_hip.so / libktx_seq.so) for decoders on an fp32 residual stream whose layers mix tokens
  * with a grouped-query sliding-window softmax attention over paged KEY and VALUE caches (partly rotated unit-RMS queries and keys,
- * values turned by their own position and results turned back by the query's, a sink in the denominator) or with a selective scan
+ * values turned by their own position and results turned back by the query's, a sink in the denominator; or un-rotated, behind a short
+ * causal convolution over time on the projections, with RMS norms over the whole q and k projections, a learned bias by distance and a
+ * window that keeps the sequence's first positions) or with a selective scan
  * (per-channel state, input-dependent step and read-out), behind RMS norms whose weight is one number, a causal convolution over
  * time on what every sublayer reads, a softmax-routed mixture whose last router outputs stand for experts that return their input,
  * and a per-layer input looked up by token.

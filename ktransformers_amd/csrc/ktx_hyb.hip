@@ -1,5 +1,6 @@
 // ktx_hyb.hip — hybrid-decoder kernels behind include/ktx_hyb.h: layer norm with bias, the sigmoid-gated post-normed residual update
-// (with the mixture's weighted gather folded in), PolyNorm, the gated delta rule (convolution + unit vectors + decay prep, state update,
+// (with the mixture's weighted gather folded in), the post-norm on a scaled residual with a depth-weighted average over a stack of
+// layer results, PolyNorm, the bounded GLU activation and a sigmoid output gate, the gated delta rule (convolution + unit vectors + decay prep, state update,
 // token-by-token recurrence on register-resident state slices), sliding-window softmax attention with a sink over a paged latent cache,
 // the sigmoid top-k router with its expert sort, and a grouped GEMM (per-head products and per-expert products) on the matrix cores.
 //

@@ -1,6 +1,7 @@
 // ktx_swa.hip — kernels behind include/ktx_swa.h: the residual update with a scalar-weight RMS norm and the rows an input convolution
 // reads, the input convolution over time, grouped-query sliding-window attention over paged key and value caches with rotated values
-// and a sink (prep, a vector-ALU form for any sizes, a matrix-core form for bf16 caches, the key-range merge), the selective scan with
+// and a sink (prep — rotating, or convolving the projections over time and norming them whole —, a vector-ALU form for any sizes, a
+// matrix-core form for bf16 caches, both with an optional bias by distance and kept first positions, the key-range merge), the selective scan with
 // its short convolution, and the softmax router with a choice correction.
 //
 // Everything a norm, an angle, a score, a router or a recurrence touches is fp32; element types only select how weights, activations
